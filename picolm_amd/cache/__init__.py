@@ -48,6 +48,7 @@ class KVGroupSpec:
     head_dim: int
     window: int = 0            # 0: all keys are kept; w > 0: the last w keys
     v_head_dim: int = 0        # size of a value where it is not that of a key
+    keeps_all: bool = False    # with a window: no ring, every key stays where it was written
 
     @property
     def value_dim(self) -> int:

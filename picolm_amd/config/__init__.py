@@ -1,11 +1,12 @@
 from .begopel import BegopelConfig
 from .llama import ConfigError, LlamaConfig, RopeScaling
+from .satedra import SatedraConfig
 from .zarinex import ZarinexConfig
 from .registry import (Architecture, architecture_name, import_architecture_modules, known_architectures, read_config_json,
                        register_architecture, resolve, unregister_architecture)
 
 __all__ = [
-    "BegopelConfig", "ZarinexConfig", "ConfigError", "LlamaConfig", "RopeScaling", "Architecture", "architecture_name", "import_architecture_modules",
+    "BegopelConfig", "SatedraConfig", "ZarinexConfig", "ConfigError", "LlamaConfig", "RopeScaling", "Architecture", "architecture_name", "import_architecture_modules",
     "known_architectures", "read_config_json", "register_architecture", "resolve",
     "unregister_architecture",
 ]

@@ -112,7 +112,9 @@ int picolm_kv_page_order(int dt, int d, int32_t* k_idx, int32_t* v_idx);
 // or null is "none"): values of a size of their own, a bias by distance added to the scaled score
 // (bias[head][min(n, bias_rows - 1)] for a key n positions back), a sink (exp(sink[head]) is one more term
 // of the softmax's denominator and adds nothing to the numerator), and a gate (the output of head h is
-// multiplied by sigmoid(gate[token * gate_stride + h * v_head_dim + c]), float rows).
+// multiplied by sigmoid(gate[token * gate_stride + h * v_head_dim + c]), float rows), and a window
+// of the operation's own (mask_window > 0: a query sees that many keys, no more than the `window`
+// that the pages and the decode step's work list are laid out for; zero: `window` itself).
 typedef struct {
     int32_t v_head_dim;
     const float* bias;
@@ -120,6 +122,7 @@ typedef struct {
     const float* sink;
     const float* gate;
     int32_t gate_stride;
+    int32_t mask_window;
 } picolm_attn_extras;
 // picolm_attn_prefill_generic / picolm_attn_decode_generic over pages kept as plain arrays K[64][d],
 // V^T[dv][64] whatever the dtype and head size, with the extras above; out rows are [H][dv] and the
@@ -134,18 +137,19 @@ int picolm_attn_decode_plain(const void* q, const void* k_pages, const void* v_p
                              const int32_t* page_table, int max_pages, int ring_pages, int H, int G, int d, int window, float scale,
                              const picolm_attn_extras* x, hipStream_t stream);
 // The same on the matrix cores: bfloat16, keys and values of the sizes that picolm_attn_plain_mfma_takes
-// says, prefill tiles of picolm_attn_plain_mfma_tile_rows() rows, no window; the caller's pages are in the
+// says, prefill tiles of picolm_attn_plain_mfma_tile_rows() rows; the caller's pages are in the
 // order of the MFMA operands (attention.h: k_page_offset(key, i, d, true), v_page_offset(i, key, dv, true)).
 int picolm_attn_plain_mfma_takes(int d, int dv);
 int picolm_attn_plain_mfma_tile_rows(void);
 int picolm_attn_prefill_plain_mfma(const void* q, const void* k_pages, const void* v_pages, void* out, const int32_t* tile_seq,
                                    const int32_t* tile_q0, int n_tiles, const int32_t* seq_slot, const int32_t* seq_pos0,
                                    const int32_t* seq_nnew, const int32_t* cu_seqlens, const int32_t* page_table, int max_pages,
-                                   int ring_pages, int H, int G, int d, float scale, const picolm_attn_extras* x, hipStream_t stream);
+                                   int ring_pages, int H, int G, int d, int window, float scale, const picolm_attn_extras* x,
+                                   hipStream_t stream);
 int picolm_attn_decode_plain_mfma(const void* q, const void* k_pages, const void* v_pages, void* out, float* partial, int n_seq,
                                   const int32_t* chunk_list, int n_chunks, int pages_per_chunk, int max_splits, const int32_t* seq_pos0,
-                                  const int32_t* page_table, int max_pages, int ring_pages, int H, int G, int d, float scale,
-                                  const picolm_attn_extras* x, hipStream_t stream);
+                                  const int32_t* page_table, int max_pages, int ring_pages, int H, int G, int d, int window,
+                                  float scale, const picolm_attn_extras* x, hipStream_t stream);
 int picolm_attn_prefill_tile_rows(void);
 int picolm_attn_prefill_generic(const void* q, const void* k_pages, const void* v_pages, void* out,
                                 int dt, const int32_t* tile_seq, const int32_t* tile_q0, int n_tiles,

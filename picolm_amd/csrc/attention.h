@@ -52,7 +52,14 @@ struct AttnArgs {
     // group) over all keys, so that they read the same keys and values at about the same time;
     // zero: they take one head's keys in turn
     int waves_take_heads;
+    // a query sees the last `mask_window` keys, fewer than the `window` that the cache entry's pages
+    // and the decode step's work list are laid out for (several layers with windows of their own
+    // may read one entry); zero: `window` itself
+    int mask_window;
 };
+
+// how many keys back a query sees (0: all)
+__device__ __forceinline__ int seen_window(const AttnArgs& a) { return a.mask_window > 0 ? a.mask_window : a.window; }
 
 // ---- the order of a page's elements ---------------------------------------------------------
 // A page holds, per KV group, the keys K[64][d] and the values transposed V^T[d][64].  Pages of

@@ -72,7 +72,8 @@ __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
     // visible key range of the tile: [lo, hi]
     const int qpos_first = row_qpos[0], qpos_last = row_qpos[n_rows - 1];
     const int hi = qpos_last;
-    const int lo = a.window > 0 ? max(0, qpos_first - a.window + 1) : 0;
+    const int seen = seen_window(a);
+    const int lo = seen > 0 ? max(0, qpos_first - seen + 1) : 0;
     int page_lo = lo / PAGE_TOKENS, page_hi = hi / PAGE_TOKENS + 1;   // [page_lo, page_hi)
     if (a.decode) {
         page_lo = work.page_lo;
@@ -138,7 +139,7 @@ __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
             for (int i = 0; i < 4; ++i) {
                 const int r = 4 * wave + i;
                 const int qp = row_qpos[r];
-                const bool vis = r < n_rows && kpos <= qp && (a.window <= 0 || qp - kpos < a.window);
+                const bool vis = r < n_rows && kpos <= qp && (seen <= 0 || qp - kpos < seen);
                 float sc = NEG_BIG;
                 if (vis) {
                     sc = s[i] * a.scale;
@@ -387,6 +388,7 @@ static void with_extras(AttnArgs& a, const picolm_attn_extras* x) {
     a.sink = x->sink;
     a.gate = x->gate;
     a.gate_stride = x->gate_stride;
+    a.mask_window = x->mask_window;
 }
 
 static int check_extras(const char* who, const picolm_attn_extras* x, int H, int d) {
@@ -395,6 +397,7 @@ static int check_extras(const char* who, const picolm_attn_extras* x, int H, int
     PICOLM_REQUIRE(!x->bias || x->bias_rows >= 1, "%s: a bias by distance needs at least one row", who);
     const int dv = x->v_head_dim > 0 ? x->v_head_dim : d;
     PICOLM_REQUIRE(!x->gate || x->gate_stride >= H * dv, "%s: gate rows of %d floats for %d heads of %d", who, x->gate_stride, H, dv);
+    PICOLM_REQUIRE(x->mask_window >= 0, "%s: a window of %d keys", who, x->mask_window);
     return 0;
 }
 

@@ -1,6 +1,6 @@
 // bf16 softmax attention on the matrix cores over pages that the caller keeps in the order of the
 // MFMA operands (attention.h: k_page_offset(key, i, d, true), v_page_offset(i, key, dv, true)), with what the vector-ALU kernels of attention_generic.hip take beside keys and
-// values: values of a size of their own, a bias by distance, a sink and an output gate.  Head sizes
+// values: values of a size of their own, a window, a bias by distance, a sink and an output gate.  Head sizes
 // of 64, 96 and 128 on either side.
 //
 // A workgroup of PLAIN_WAVES waves per piece of work; the waves take the tiles of 32 keys in turn and
@@ -85,7 +85,7 @@ __global__ __launch_bounds__(64 * PLAIN_WAVES) void attn_plain_mfma_kernel(AttnA
         tok = a.cu_seqlens[seq] + l, qpos = pos0 + l, qpos_first = pos0 + q0;
         slot = a.seq_slot[seq];
         hi = pos0 + min(q0 + 31, nnew - 1);
-        page_lo = 0, page_hi = hi / PAGE_TOKENS + 1;
+        page_lo = decode_first_page(seen_window(a), qpos_first), page_hi = hi / PAGE_TOKENS + 1;      // (the tile's first query sees furthest back)
     }
     // the wave's queries as operands: column `col`, k-step s covers elements 16 s + 8 h .. + 8
     bf16x8 Qf[D / 16];
@@ -113,7 +113,10 @@ __global__ __launch_bounds__(64 * PLAIN_WAVES) void attn_plain_mfma_kernel(AttnA
     const int tile_hi = min(2 * page_hi, hi / 32 + 1);       // tiles of 32 keys: this wave takes tile_lo, tile_lo + PLAIN_WAVES, ... below tile_hi
     const bool keys_in_turn = !a.waves_take_heads;           // the waves share one head's keys
     const int tile_step = keys_in_turn ? PLAIN_WAVES : 1;
-    const int tile_lo = 2 * page_lo + (keys_in_turn ? wave : 0);
+    // with a window, the tile of 32 keys that holds the oldest key any query of this wave sees
+    const int seen = seen_window(a);
+    const int oldest = seen > 0 ? max(0, qpos_first - seen + 1) : 0;
+    const int tile_lo = max(2 * page_lo, oldest / 32) + (keys_in_turn ? wave : 0);
     // two sets of operands in turn: the loads of the tile after this one are queued before this
     // tile's products and stay there (the scheduler may not move them past the barrier), and the
     // page of the tile after that is looked up meanwhile
@@ -149,7 +152,7 @@ __global__ __launch_bounds__(64 * PLAIN_WAVES) void attn_plain_mfma_kernel(AttnA
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
             const int key = key0 + key_of_elem(e, h);
-            const bool vis = q_ok && key <= qpos;
+            const bool vis = q_ok && key <= qpos && (seen <= 0 || key > qpos - seen);
             S[e] = vis ? fmaf(S[e], scale2, bv[e]) : NEG_BIG;
             mx = fmaxf(mx, S[e]);
         }
@@ -285,7 +288,10 @@ static int fill_extras(const char* who, AttnArgs& a, const picolm_attn_extras* x
     if (!x) return 0;
     PICOLM_REQUIRE(!x->bias || x->bias_rows >= 1, "%s: a bias by distance needs at least one row", who);
     PICOLM_REQUIRE(!x->gate || x->gate_stride >= a.H * dv, "%s: gate rows of %d floats for %d heads of %d", who, x->gate_stride, a.H, dv);
+    PICOLM_REQUIRE(x->mask_window >= 0 && (a.window <= 0 || x->mask_window <= a.window), "%s: a window of %d keys over pages laid out for %d", who,
+                   x->mask_window, a.window);
     a.bias = x->bias, a.bias_rows = x->bias_rows, a.sink = x->sink, a.gate = x->gate, a.gate_stride = x->gate_stride;
+    a.mask_window = x->mask_window;
     return 0;
 }
 
@@ -293,13 +299,14 @@ static int fill_extras(const char* who, AttnArgs& a, const picolm_attn_extras* x
 extern "C" int picolm_attn_prefill_plain_mfma(const void* q, const void* k_pages, const void* v_pages, void* out, const int32_t* tile_seq,
                                               const int32_t* tile_q0, int n_tiles, const int32_t* seq_slot, const int32_t* seq_pos0,
                                               const int32_t* seq_nnew, const int32_t* cu_seqlens, const int32_t* page_table, int max_pages,
-                                              int ring_pages, int H, int G, int d, float scale, const picolm_attn_extras* x,
+                                              int ring_pages, int H, int G, int d, int window, float scale, const picolm_attn_extras* x,
                                               hipStream_t stream) {
     if (check_attn_sizes("attn_prefill_plain_mfma", H, G, d, max_pages, ring_pages)) return -1;
+    PICOLM_REQUIRE(window >= 0, "attn_prefill_plain_mfma: a window of %d keys", window);
     PICOLM_REQUIRE(H <= 65535, "attn_prefill_plain_mfma: %d heads exceed the grid", H);
     if (n_tiles <= 0) return 0;
     AttnArgs a = {q, k_pages, v_pages, out, nullptr, tile_seq, tile_q0, seq_slot, seq_pos0, seq_nnew,
-                  cu_seqlens, page_table, max_pages, ring_pages, H, G, d, 0, scale, 0, nullptr, 0, 1,
+                  cu_seqlens, page_table, max_pages, ring_pages, H, G, d, window, scale, 0, nullptr, 0, 1,
                   nullptr, nullptr, nullptr, nullptr, 0};
     int dv;
     if (fill_extras("attn_prefill_plain_mfma", a, x, dv)) return -1;
@@ -312,14 +319,15 @@ extern "C" int picolm_attn_prefill_plain_mfma(const void* q, const void* k_pages
 extern "C" int picolm_attn_decode_plain_mfma(const void* q, const void* k_pages, const void* v_pages, void* out, float* partial, int n_seq,
                                              const int32_t* chunk_list, int n_chunks, int pages_per_chunk, int max_splits,
                                              const int32_t* seq_pos0, const int32_t* page_table, int max_pages, int ring_pages, int H,
-                                             int G, int d, float scale, const picolm_attn_extras* x, hipStream_t stream) {
+                                             int G, int d, int window, float scale, const picolm_attn_extras* x, hipStream_t stream) {
     if (check_attn_sizes("attn_decode_plain_mfma", H, G, d, max_pages, ring_pages)) return -1;
+    PICOLM_REQUIRE(window >= 0, "attn_decode_plain_mfma: a window of %d keys", window);
     if (check_decode_chunks("attn_decode_plain_mfma", partial, chunk_list, n_chunks, pages_per_chunk, max_splits)) return -1;
     if (n_seq <= 0 || n_chunks <= 0) return 0;
     const int hc = ceil_div(H / G, 32);
     PICOLM_REQUIRE((int64_t)n_chunks * G * hc < (1ll << 31), "attn_decode_plain_mfma: %d chunks of %d waves exceed the grid", n_chunks, G * hc);
     AttnArgs a = {q, k_pages, v_pages, out, partial, nullptr, nullptr, nullptr, seq_pos0, nullptr, nullptr,
-                  page_table, max_pages, ring_pages, H, G, d, 0, scale, 1, chunk_list, pages_per_chunk, max_splits,
+                  page_table, max_pages, ring_pages, H, G, d, window, scale, 1, chunk_list, pages_per_chunk, max_splits,
                   nullptr, nullptr, nullptr, nullptr, 0};
     int dv;
     if (fill_extras("attn_decode_plain_mfma", a, x, dv)) return -1;

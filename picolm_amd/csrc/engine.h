@@ -150,8 +150,12 @@ typedef struct {
 // group keeps the last `window` keys of a sequence in a ring of pages (enough for a window and a
 // prefill chunk of 256 tokens); 0: all keys.  v_head_dim: the size of a value where it is not that
 // of a key (0: the same); the ATTENTION operation takes one size for both, a called operation any.
+// keeps_all = 1 with a window: every key stays in its page (no ring) and the window only bounds
+// what a query's work list and tiles visit; a called operation on such a group sees steps of any
+// length.
 typedef struct {
     int32_t n_entries, n_kv_heads, head_dim, window, v_head_dim;
+    int32_t keeps_all;
 } picolm_kv_group;
 
 // Fixed-size state per sequence for `n_entries` layer calls, zeroed when a slot is given out.

@@ -569,7 +569,7 @@ extern "C" int picolm_engine_create(const picolm_program* program, int64_t max_t
         g.max_pages = e->max_pages;
         // a window's ring: the window of the first query of a chunk of new tokens together with the
         // whole chunk, which is written before its queries are answered
-        g.ring_pages = g.spec.window > 0 ? std::min(pages_for(g.spec.window - 1 + WINDOW_STEP_TOKENS) + 1, e->max_pages) : e->max_pages;
+        g.ring_pages = g.spec.window > 0 && !g.spec.keeps_all ? std::min(pages_for(g.spec.window - 1 + WINDOW_STEP_TOKENS) + 1, e->max_pages) : e->max_pages;
         g.n_pages = (int)std::min<int64_t>(n_pages, (int64_t)e->n_slots * g.ring_pages);
         g.pool.init(g.n_pages);
         g.pages.assign(e->n_slots, {});

@@ -43,6 +43,8 @@ typedef struct {
     const float* bias;       // [H][bias_rows] by distance, the last entry for every distance beyond; null: none
     int32_t bias_rows;
     const float* sink;       // [H] or null
+    int32_t window;          // > 0: a query sees its last `window` keys, no more than the cache entry's own window (which
+                             // bounds the pages a step visits); 0: what the cache entry's window says
 } picolm_sink_attention_args;
 int picolm_call_sink_attention(void* user, const picolm_step_view* v);
 
@@ -111,7 +113,7 @@ typedef struct {
 int picolm_call_normed_sum(void* user, const picolm_step_view* v);
 
 // out <- f(in) element by element over rows [width] (`in` absent: in place, one dtype):
-//   kind 1: max(x, 0)^2;  kind 2: param tanh(x / param)
+//   kind 1: max(x, 0)^2;  kind 2: param tanh(x / param);  kind 3: param x
 typedef struct {
     int32_t kind, width;
     int32_t in_dtype, out_dtype;     // PICOLM_F32 / PICOLM_BF16
@@ -143,7 +145,8 @@ typedef struct {
 int picolm_call_token_shift(void* user, const picolm_step_view* v);
 
 // out[c] = x[c] * act(g[c] + bias[c]) over `width` columns; act 0: no gate (a copy into another
-// dtype or stride), 1: silu, 2: sigmoid.
+// dtype or stride), 1: silu, 2: sigmoid.  g_per_row = 1: one gate a row, the float at g_off, for
+// every column (no bias then).
 //   in: x rows [x_stride] of x_dtype, columns at x_off; extra[0]: g float rows [g_stride], columns at
 //   g_off (act > 0); out: rows [width] of out_dtype.
 typedef struct {
@@ -152,6 +155,7 @@ typedef struct {
     int32_t g_stride, g_off;
     int32_t out_dtype;
     const float* bias;       // [width] or null
+    int32_t g_per_row;
 } picolm_gate_rows_args;
 int picolm_call_gate_rows(void* user, const picolm_step_view* v);
 
@@ -167,9 +171,11 @@ int picolm_call_slice_norm(void* user, const picolm_step_view* v);
 
 // A product per head: out[h] = W_h in[h] (transposed = 0: W [heads out_dim][in_dim]) or
 // out[h] = W_h^T in[h] (transposed = 1: W [heads in_dim][out_dim]), float accumulation, and then
-// out *= act(g) with g at the output's columns (gate_act 0: none, 1 silu, 2 sigmoid).
-//   in: rows [in_stride] of in_dtype, heads side by side at in_off; out: rows [out_stride] of
-//   out_dtype, heads side by side at out_off; extra[0]: g float rows [gate_stride], at gate_off.
+// out *= act(g) with g at the output's columns (gate_act 0: none, 1 silu, 2 sigmoid), or with
+// gate_per_head = 1 one g a head, head h's at gate_off + h.
+//   in: rows [in_stride] of in_dtype, head h at in_off + h in_head_stride; out: rows [out_stride] of
+//   out_dtype, head h at out_off + h out_head_stride (a head stride of 0: the heads lie side by
+//   side, in_dim or out_dim apart); extra[0]: g float rows [gate_stride], at gate_off.
 typedef struct {
     const void* weight;
     int32_t weight_dt;       // PICOLM_F32 / PICOLM_BF16
@@ -177,6 +183,7 @@ typedef struct {
     int32_t in_stride, in_off, in_dtype;
     int32_t out_stride, out_off, out_dtype;
     int32_t gate_act, gate_stride, gate_off;
+    int32_t in_head_stride, out_head_stride, gate_per_head;
 } picolm_head_linear_args;
 int picolm_call_head_linear(void* user, const picolm_step_view* v);
 
@@ -225,19 +232,55 @@ typedef struct {
 } picolm_decay_scan_args;
 int picolm_call_decay_scan(void* user, const picolm_step_view* v);
 
+// Layer norm with a weight and an optional bias: out = (x - mean) / sqrt(var + eps) * weight + bias,
+// var the mean of the squared deviations, all in float.
+//   in: x float rows [width]; out: rows [width] of out_dtype.  gathers = 1: the operation covers the
+//   wanted rows, and row i reads the row of x that the step's want_rows[i] names.
+typedef struct {
+    const float* weight;     // [width]
+    const float* bias;       // [width] or null
+    int32_t width, out_dtype;
+    float eps;
+    int32_t gathers;
+} picolm_layer_norm_args;
+int picolm_call_layer_norm(void* user, const picolm_step_view* v);
+
+// Rotation by position of `heads` stretches of a row: of each stretch's first `dims` entries, entry
+// i < dims / 2 is paired with entry i + dims / 2 (half = 1) or entry 2i with 2i + 1 (half = 0); the
+// pair (u, v) of a token at position p becomes (u cos - v sin, v cos + u sin) with
+// cos = cos_table[p][i], sin = sin_table[p][i]; the stretch's other entries are copied.
+//   in: float rows [in_stride], stretch h at in_off + h in_head_stride; out: float rows
+//   [out_stride], stretch h at out_off + h out_head_stride (in place: out names the same buffer,
+//   and the offsets and strides are equal).
+typedef struct {
+    const float* cos_table;  // [table_positions][dims / 2]
+    const float* sin_table;
+    int32_t table_positions, dims, half, heads, width;      // width: entries of a stretch, >= dims
+    int32_t in_stride, in_off, in_head_stride;
+    int32_t out_stride, out_off, out_head_stride;
+} picolm_rotate_heads_args;
+int picolm_call_rotate_heads(void* user, const picolm_step_view* v);
+
 // ---- a routed feed-forward ---------------------------------------------------------------------
-// Each row picks the `top` experts with the largest logits (ties: the lower index), weighted by
-// the softmax over the picked logits.
-//   in: float rows [experts] of router logits without bias; out: rows of 2 top words: the picked
-//   experts (int32) and then their weights (float).
+// Each row picks `top` of its `experts` router outputs (ties: the lower index).
+//   scoring 0: the largest logits + bias are picked, weighted by the softmax over the picked
+//              (biased) logits alone;
+//   scoring 1: s = softmax over all the logits; the largest s + bias are picked; the weights are
+//              the picked s over their sum (+ 1e-20), times `scale`.
+//   in: float rows [in_stride] (0: experts) whose first `experts` entries are the router logits
+//   without bias; out: rows of 2 top words: the picked outputs (int32) and then their weights (float).
 typedef struct {
     const float* bias;       // [experts] or null
     int32_t experts, top;
+    int32_t scoring, in_stride;
+    float scale;             // scoring 1
 } picolm_route_top_args;
 int picolm_call_route_top(void* user, const picolm_step_view* v);
 
 // The picked experts of every row: y[t][k] = W_down[e] (silu(W_gate[e] h) * (W_up[e] h)), e the k-th
-// pick of row t, and their weighted sum  out[t] = sum_k w[t][k] y[t][k] (+ out[t] if `adds`).
+// pick of row t, and their weighted sum  out[t] = sum_k w[t][k] y[t][k] (+ out[t] if `adds`).  A pick
+// e with experts <= e < experts + identity stands for an expert that gives its input back:
+// y[t][k] = h[t]; such picks read no weights.
 //   in: h rows [width] in the engine's dtype; extra[0]: the picks as route_top leaves them; extra[1]:
 //   scratch float rows [top ff]; out: float rows [width].  With extra[2], scratch float rows
 //   [top width], and extra[3], scratch rows of top + experts + 1 words, a step of many rows in
@@ -249,6 +292,7 @@ typedef struct {
     int32_t weight_dt;
     int32_t experts, top, width, ff;
     int32_t adds;            // 1: out += the sum; 0: out = the sum
+    int32_t identity;        // picks from `experts` up to experts + identity give the row itself
 } picolm_routed_experts_args;
 int picolm_call_routed_experts(void* user, const picolm_step_view* v);
 

@@ -96,8 +96,8 @@ extern "C" int picolm_call_sink_attention(void* user, const picolm_step_view* v)
                    "sink_attention: buffers or the cache entry are missing");
     const int H = a->n_heads, G = a->n_kv_heads, d = a->head_dim, dv = a->v_head_dim, dt = v->dtype, es = elem_bytes(dt);
     PICOLM_REQUIRE(H > 0 && G > 0 && H % G == 0 && d > 0 && dv > 0, "sink_attention: %d heads over %d, sizes %d and %d", H, G, d, dv);
-    PICOLM_REQUIRE(G == v->n_kv_heads && d == v->head_dim && dv == v->v_head_dim && v->window == 0,
-                   "sink_attention: the cache entry holds %d heads of %d and %d (window %d), the operation has %d of %d and %d and none", v->n_kv_heads,
+    PICOLM_REQUIRE(G == v->n_kv_heads && d == v->head_dim && dv == v->v_head_dim && v->window >= 0,
+                   "sink_attention: the cache entry holds %d heads of %d and %d (window %d), the operation has %d of %d and %d", v->n_kv_heads,
                    v->head_dim, v->v_head_dim, v->window, G, d, dv);
     PICOLM_REQUIRE(v->in_row_bytes >= a->in_stride * 4 && a->q_off >= 0 && a->q_off + H * d <= a->in_stride && a->k_off >= 0 &&
                        a->k_off + G * d <= a->in_stride && a->v_off >= 0 && a->v_off + G * dv <= a->in_stride &&
@@ -105,6 +105,8 @@ extern "C" int picolm_call_sink_attention(void* user, const picolm_step_view* v)
                    "sink_attention: the input rows of %d floats do not hold what the offsets name", a->in_stride);
     PICOLM_REQUIRE(v->out_row_bytes >= H * dv * es && v->extra_row_bytes[0] >= H * d * es, "sink_attention: output or scratch rows too short");
     PICOLM_REQUIRE(!v->kv_writes || v->write_pages, "sink_attention: no pages to write to");
+    PICOLM_REQUIRE(a->window >= 0 && (v->window <= 0 || a->window <= v->window), "sink_attention: a window of %d keys over a cache entry laid out for %d",
+                   a->window, v->window);
     PICOLM_REQUIRE(H + G + G <= 65535, "sink_attention: %d heads exceed the grid", H + 2 * G);
     if (v->n_tokens <= 0) return 0;
     const float* in = (const float*)v->in;
@@ -126,25 +128,26 @@ extern "C" int picolm_call_sink_attention(void* user, const picolm_step_view* v)
     x.sink = a->sink;
     x.gate = a->gate_off >= 0 ? in + a->gate_off : nullptr;
     x.gate_stride = a->in_stride;
+    x.mask_window = a->window;
     if (mfma && v->is_decode)
         return picolm_attn_decode_plain_mfma(v->extra[0], v->k_pages, v->v_pages, v->out, v->partial, v->n_seq, v->chunk_list, v->n_chunks,
                                              v->pages_per_chunk, v->most_chunks, v->seq_pos0, v->page_table, v->max_pages, v->ring_pages, H,
-                                             G, d, a->scale, &x, v->stream);
+                                             G, d, v->window, a->scale, &x, v->stream);
     if (mfma) {
         PICOLM_REQUIRE(v->tile_seq && v->tile_rows == picolm_attn_plain_mfma_tile_rows(), "sink_attention: the step has no tiles of %d rows",
                        picolm_attn_plain_mfma_tile_rows());
         return picolm_attn_prefill_plain_mfma(v->extra[0], v->k_pages, v->v_pages, v->out, v->tile_seq, v->tile_q0, v->n_tiles, v->seq_slot,
                                               v->seq_pos0, v->seq_nnew, v->cu_seqlens, v->page_table, v->max_pages, v->ring_pages, H, G, d,
-                                              a->scale, &x, v->stream);
+                                              v->window, a->scale, &x, v->stream);
     }
     if (v->is_decode)
         return picolm_attn_decode_plain(v->extra[0], v->k_pages, v->v_pages, v->out, v->partial, dt, v->n_seq, v->chunk_list, v->n_chunks,
                                         v->pages_per_chunk, v->most_chunks, v->seq_pos0, v->page_table, v->max_pages, v->ring_pages, H, G, d,
-                                        0, a->scale, &x, v->stream);
+                                        v->window, a->scale, &x, v->stream);
     PICOLM_REQUIRE(v->tile_seq && v->tile_rows == picolm_attn_prefill_tile_rows(), "sink_attention: the step has no tiles of %d rows",
                    picolm_attn_prefill_tile_rows());
     return picolm_attn_prefill_plain(v->extra[0], v->k_pages, v->v_pages, v->out, dt, v->tile_seq, v->tile_q0, v->n_tiles, v->seq_slot,
-                                     v->seq_pos0, v->seq_nnew, v->cu_seqlens, v->page_table, v->max_pages, v->ring_pages, H, G, d, 0,
+                                     v->seq_pos0, v->seq_nnew, v->cu_seqlens, v->page_table, v->max_pages, v->ring_pages, H, G, d, v->window,
                                      a->scale, &x, v->stream);
 }
 
@@ -719,6 +722,8 @@ __global__ void map_rows_kernel(const TI* __restrict__ in, TO* __restrict__ out,
             y = p * p;
         } else if (kind == 2) {
             y = param * tanhf(x / param);
+        } else if (kind == 3) {
+            y = param * x;
         }
         out[i] = from_f32<TO>(y);
     }
@@ -727,7 +732,7 @@ __global__ void map_rows_kernel(const TI* __restrict__ in, TO* __restrict__ out,
 extern "C" int picolm_call_map_rows(void* user, const picolm_step_view* v) {
     const picolm_map_rows_args* a = (const picolm_map_rows_args*)user;
     VIEW_REQUIRE("map_rows", v);
-    PICOLM_REQUIRE(a && v->out && a->width > 0 && (a->kind == 1 || (a->kind == 2 && a->param > 0.f)), "map_rows: kind %d over a width of %d",
+    PICOLM_REQUIRE(a && v->out && a->width > 0 && (a->kind == 1 || (a->kind == 2 && a->param > 0.f) || a->kind == 3), "map_rows: kind %d over a width of %d",
                    a ? a->kind : -1, a ? a->width : 0);
     PICOLM_REQUIRE((a->in_dtype == PICOLM_F32 || a->in_dtype == PICOLM_BF16) && (a->out_dtype == PICOLM_F32 || a->out_dtype == PICOLM_BF16),
                    "map_rows: unknown dtype");

@@ -23,13 +23,37 @@ static inline int elem_bytes(int dt) { return dt == PICOLM_F32 ? 4 : 2; }
 
 // ---- the pick --------------------------------------------------------------------------------------
 // a thread a row; the picks come out in the order (logit falling, index rising)
-__global__ void route_top_kernel(const float* __restrict__ logits, const float* __restrict__ bias, int32_t* __restrict__ out, int E, int top,
-                                 int n_rows) {
+__global__ void route_top_kernel(const float* __restrict__ logits, int in_stride, const float* __restrict__ bias, int32_t* __restrict__ out, int E,
+                                 int top, int n_rows, int scoring, float scale) {
     const int row = blockIdx.x * blockDim.x + threadIdx.x;
     if (row >= n_rows) return;
-    const float* z = logits + (size_t)row * E;
+    const float* z = logits + (size_t)row * in_stride;
     int32_t* ids = out + (size_t)row * 2 * top;
     float* w = (float*)(ids + top);
+    if (scoring == 1) {
+        // s = softmax over every output; the picks are the largest s + bias, their weights the picked s over their sum
+        float zmax = -INFINITY, den = 0.f;
+        for (int e = 0; e < E; ++e) zmax = fmaxf(zmax, z[e]);
+        for (int e = 0; e < E; ++e) den += expf(z[e] - zmax);
+        float last_c = INFINITY, sum = 0.f;
+        int last_e = -1;
+        for (int k = 0; k < top; ++k) {
+            float best = -INFINITY, best_s = 0.f;
+            int be = -1;
+            for (int e = 0; e < E; ++e) {
+                const float se = expf(z[e] - zmax) / den, ce = se + (bias ? bias[e] : 0.f);
+                const bool after_last = ce < last_c || (ce == last_c && e > last_e);
+                if (after_last && (be < 0 || ce > best)) best = ce, be = e, best_s = se;
+            }
+            if (be < 0) be = k % E, best = -INFINITY, best_s = 0.f;     // (only logits that are no numbers lead here)
+            ids[k] = be;
+            w[k] = best_s;
+            sum += best_s;
+            last_c = best, last_e = be;
+        }
+        for (int k = 0; k < top; ++k) w[k] = w[k] / (sum + 1e-20f) * scale;
+        return;
+    }
     float last_z = INFINITY, first_z = 0.f, sum = 0.f;
     int last_e = -1;
     for (int k = 0; k < top; ++k) {
@@ -56,9 +80,12 @@ extern "C" int picolm_call_route_top(void* user, const picolm_step_view* v) {
     VIEW_REQUIRE("route_top", v);
     PICOLM_REQUIRE(a && v->in && v->out && a->experts > 0 && a->top > 0 && a->top <= a->experts, "route_top: %d picks among %d experts",
                    a ? a->top : 0, a ? a->experts : 0);
-    PICOLM_REQUIRE(v->in_row_bytes >= a->experts * 4 && v->out_row_bytes >= 2 * a->top * 4, "route_top: rows too short");
+    const int in_stride = a->in_stride ? a->in_stride : a->experts;
+    PICOLM_REQUIRE(in_stride >= a->experts && v->in_row_bytes >= (int64_t)in_stride * 4 && v->out_row_bytes >= 2 * a->top * 4, "route_top: rows too short");
+    PICOLM_REQUIRE(a->scoring == 0 || a->scoring == 1, "route_top: scoring %d is not known", a->scoring);
     if (v->rows <= 0) return 0;
-    route_top_kernel<<<ceil_div(v->rows, 64), 64, 0, v->stream>>>((const float*)v->in, a->bias, (int32_t*)v->out, a->experts, a->top, v->rows);
+    route_top_kernel<<<ceil_div(v->rows, 64), 64, 0, v->stream>>>((const float*)v->in, in_stride, a->bias, (int32_t*)v->out, a->experts, a->top,
+                                                                 v->rows, a->scoring, a->scale);
     PICOLM_LAUNCH_CHECK("route_top");
     return 0;
 }
@@ -125,9 +152,18 @@ __global__ __launch_bounds__(256) void expert_hidden_kernel(const TH* __restrict
 }
 
 // out[row][d] (+)= sum_k w[row][k] (W_down[e_k][d] . act[row][k])
-template <typename TW>
+// a row's picks that stand for "the input itself": the sum of their weights
+__device__ __forceinline__ float identity_weight(const int32_t* ids, const float* w, int top, int E, int identity) {
+    float total = 0.f;
+    for (int k = 0; k < top; ++k)
+        if (ids[k] >= E && ids[k] < E + identity) total += w[k];
+    return total;
+}
+
+template <typename TW, typename TH>
 __global__ __launch_bounds__(256) void expert_down_kernel(const float* __restrict__ act, const int32_t* __restrict__ picks, float* __restrict__ out,
-                                                          const TW* __restrict__ down, int E, int top, int D, int F, int adds) {
+                                                          const TW* __restrict__ down, int E, int top, int D, int F, int adds,
+                                                          const TH* __restrict__ h, int identity) {
     extern __shared__ float moe_lds[];       // [top][F]
     const int row = blockIdx.x;
     for (int c = threadIdx.x; c < top * F; c += blockDim.x) moe_lds[c] = act[(size_t)row * top * F + c];
@@ -146,9 +182,13 @@ __global__ __launch_bounds__(256) void expert_down_kernel(const float* __restric
 #pragma unroll
         for (int j = 0; j < 4; ++j) total[j] += w[k] * wave_sum(part[j]);
     }
+    const float same = identity > 0 ? identity_weight(ids, w, top, E, identity) : 0.f;
 #pragma unroll
     for (int j = 0; j < 4; ++j)
-        if (lane == 0 && d0 + j < D) out[(size_t)row * D + d0 + j] = (adds ? out[(size_t)row * D + d0 + j] : 0.f) + total[j];
+        if (lane == 0 && d0 + j < D) {
+            const size_t at = (size_t)row * D + d0 + j;
+            out[at] = (adds ? out[at] : 0.f) + total[j] + (same != 0.f ? same * to_f32<TH>(h[at]) : 0.f);
+        }
 }
 
 // ---- the same for many rows, on the matrix cores ------------------------------------------------------
@@ -291,15 +331,16 @@ __global__ __launch_bounds__(256) void grouped_tile_kernel(const bf16_t* __restr
 
 // out[row] (+)= sum_k w[row][k] y[row][k], in the order of the picks
 __global__ void grouped_sum_kernel(const float* __restrict__ y, const int32_t* __restrict__ picks, float* __restrict__ out, int E, int top, int D,
-                                   int adds) {
+                                   int adds, const bf16_t* __restrict__ h, int identity) {
     const size_t row = blockIdx.x;
     const int32_t* ids = picks + row * 2 * top;
     const float* w = (const float*)(ids + top);
+    const float same = identity > 0 ? identity_weight(ids, w, top, E, identity) : 0.f;
     for (int d = threadIdx.x; d < D; d += blockDim.x) {
         float total = 0.f;
         for (int k = 0; k < top; ++k)
             if (ids[k] >= 0 && ids[k] < E) total += w[k] * y[(row * top + k) * D + d];
-        out[row * D + d] = (adds ? out[row * D + d] : 0.f) + total;
+        out[row * D + d] = (adds ? out[row * D + d] : 0.f) + total + (same != 0.f ? same * bf16_bits_to_f32(h[row * D + d]) : 0.f);
     }
 }
 
@@ -310,7 +351,7 @@ extern "C" int picolm_call_routed_experts(void* user, const picolm_step_view* v)
     VIEW_REQUIRE("routed_experts", v);
     PICOLM_REQUIRE(a && a->gate && a->up && a->down && v->in && v->out && v->extra[0] && v->extra[1], "routed_experts: weights or buffers are missing");
     const int E = a->experts, top = a->top, D = a->width, F = a->ff;
-    PICOLM_REQUIRE(E > 0 && top > 0 && top <= E && D > 0 && F > 0 && (a->weight_dt == PICOLM_F32 || a->weight_dt == PICOLM_BF16),
+    PICOLM_REQUIRE(E > 0 && top > 0 && a->identity >= 0 && top <= E + a->identity && D > 0 && F > 0 && (a->weight_dt == PICOLM_F32 || a->weight_dt == PICOLM_BF16),
                    "routed_experts: %d picks among %d experts of %d to %d", top, E, D, F);
     PICOLM_REQUIRE(v->dtype == PICOLM_BF16 || a->weight_dt == PICOLM_F32, "routed_experts: the 32-bit engine takes 32-bit weights");
     PICOLM_REQUIRE(v->in_row_bytes >= D * elem_bytes(v->dtype) && v->out_row_bytes >= D * 4 && v->extra_row_bytes[0] >= 2 * top * 4 &&
@@ -340,7 +381,7 @@ extern "C" int picolm_call_routed_experts(void* user, const picolm_step_view* v)
         grouped_tile_kernel<false><<<dim3(tiles, ceil_div(D, GM_COLS)), 256, 0, v->stream>>>((const bf16_t*)act, plan, y, (const bf16_t*)a->down,
                                                                                             nullptr, E, top, F, D);
         PICOLM_LAUNCH_CHECK("routed_experts (down, grouped)");
-        grouped_sum_kernel<<<v->rows, 256, 0, v->stream>>>(y, picks, (float*)v->out, E, top, D, a->adds);
+        grouped_sum_kernel<<<v->rows, 256, 0, v->stream>>>(y, picks, (float*)v->out, E, top, D, a->adds, (const bf16_t*)v->in, a->identity);
         PICOLM_LAUNCH_CHECK("routed_experts (sum)");
         return 0;
     }
@@ -349,17 +390,20 @@ extern "C" int picolm_call_routed_experts(void* user, const picolm_step_view* v)
         expert_hidden_kernel<float, float><<<grid_a, 256, lds_a, v->stream>>>((const float*)v->in, picks, act, (const float*)a->gate,
                                                                               (const float*)a->up, E, top, D, F);
         PICOLM_LAUNCH_CHECK("routed_experts (hidden)");
-        expert_down_kernel<float><<<grid_b, 256, lds_b, v->stream>>>(act, picks, (float*)v->out, (const float*)a->down, E, top, D, F, a->adds);
+        expert_down_kernel<float, float><<<grid_b, 256, lds_b, v->stream>>>(act, picks, (float*)v->out, (const float*)a->down, E, top, D, F, a->adds,
+                                                                            (const float*)v->in, a->identity);
     } else if (a->weight_dt == PICOLM_F32) {
         expert_hidden_kernel<float, bf16_t><<<grid_a, 256, lds_a, v->stream>>>((const bf16_t*)v->in, picks, act, (const float*)a->gate,
                                                                                (const float*)a->up, E, top, D, F);
         PICOLM_LAUNCH_CHECK("routed_experts (hidden)");
-        expert_down_kernel<float><<<grid_b, 256, lds_b, v->stream>>>(act, picks, (float*)v->out, (const float*)a->down, E, top, D, F, a->adds);
+        expert_down_kernel<float, bf16_t><<<grid_b, 256, lds_b, v->stream>>>(act, picks, (float*)v->out, (const float*)a->down, E, top, D, F, a->adds,
+                                                                             (const bf16_t*)v->in, a->identity);
     } else {
         expert_hidden_kernel<bf16_t, bf16_t><<<grid_a, 256, lds_a, v->stream>>>((const bf16_t*)v->in, picks, act, (const bf16_t*)a->gate,
                                                                                 (const bf16_t*)a->up, E, top, D, F);
         PICOLM_LAUNCH_CHECK("routed_experts (hidden)");
-        expert_down_kernel<bf16_t><<<grid_b, 256, lds_b, v->stream>>>(act, picks, (float*)v->out, (const bf16_t*)a->down, E, top, D, F, a->adds);
+        expert_down_kernel<bf16_t, bf16_t><<<grid_b, 256, lds_b, v->stream>>>(act, picks, (float*)v->out, (const bf16_t*)a->down, E, top, D, F, a->adds,
+                                                                              (const bf16_t*)v->in, a->identity);
     }
     PICOLM_LAUNCH_CHECK("routed_experts (down)");
     return 0;

@@ -107,13 +107,13 @@ extern "C" int picolm_call_token_shift(void* user, const picolm_step_view* v) {
 
 // ---- a gate over columns ---------------------------------------------------------------------------
 __global__ void gate_rows_kernel(const void* __restrict__ x, int x_stride, int x_off, int x_dt, const float* __restrict__ g, int g_stride,
-                                 int g_off, const float* __restrict__ bias, void* __restrict__ out, int out_dt, int W, int act, int64_t n) {
+                                 int g_off, const float* __restrict__ bias, void* __restrict__ out, int out_dt, int W, int act, int64_t n, int g_per_row) {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
         const size_t row = i / W;
         const int c = (int)(i % W);
         float y = load_as_f32(x, row * x_stride + x_off + c, x_dt);
         if (act) {
-            const float z = g[row * g_stride + g_off + c] + (bias ? bias[c] : 0.f);
+            const float z = g_per_row ? g[row * g_stride + g_off] : g[row * g_stride + g_off + c] + (bias ? bias[c] : 0.f);
             y *= act == 1 ? silu_f(z) : sigmoid_f(z);
         }
         store_from_f32(out, (size_t)i, out_dt, y);
@@ -128,13 +128,14 @@ extern "C" int picolm_call_gate_rows(void* user, const picolm_step_view* v) {
     PICOLM_REQUIRE(a->x_off >= 0 && a->x_off + a->width <= a->x_stride && v->in_row_bytes >= a->x_stride * elem_bytes(a->x_dtype) &&
                        v->out_row_bytes >= a->width * elem_bytes(a->out_dtype),
                    "gate_rows: rows too short for %d columns at %d of %d", a->width, a->x_off, a->x_stride);
-    PICOLM_REQUIRE(!a->act || (v->extra[0] && a->g_off >= 0 && a->g_off + a->width <= a->g_stride && v->extra_row_bytes[0] >= a->g_stride * 4),
+    PICOLM_REQUIRE(!a->act || (v->extra[0] && a->g_off >= 0 && a->g_off + (a->g_per_row ? 1 : a->width) <= a->g_stride &&
+                               v->extra_row_bytes[0] >= a->g_stride * 4 && !(a->g_per_row && a->bias)),
                    "gate_rows: the gate's rows of %d floats do not hold %d at %d", a->g_stride, a->width, a->g_off);
     if (v->rows <= 0) return 0;
     const int64_t n = (int64_t)v->rows * a->width;
     const unsigned blocks = (unsigned)std::min<int64_t>(ceil_div64(n, 256), 65536);
     gate_rows_kernel<<<blocks, 256, 0, v->stream>>>(v->in, a->x_stride, a->x_off, a->x_dtype, (const float*)v->extra[0], a->g_stride, a->g_off,
-                                                   a->bias, v->out, a->out_dtype, a->width, a->act, n);
+                                                   a->bias, v->out, a->out_dtype, a->width, a->act, n, a->g_per_row);
     PICOLM_LAUNCH_CHECK("gate_rows");
     return 0;
 }
@@ -183,19 +184,20 @@ __global__ __launch_bounds__(256) void head_linear_kernel(picolm_head_linear_arg
     extern __shared__ float hl_in[];      // [HL_ROWS][in_dim] | partial sums [4][HL_ROWS][HL_COLS] (transposed)
     const int head = blockIdx.y, row0 = blockIdx.x * HL_ROWS, nr = min(HL_ROWS, n_rows - row0);
     const int K = a.in_dim, N = a.out_dim, o0 = blockIdx.z * HL_COLS;
+    const size_t in_head = (size_t)head * (a.in_head_stride ? a.in_head_stride : K), out_head = (size_t)head * (a.out_head_stride ? a.out_head_stride : N);
     for (int idx = threadIdx.x; idx < HL_ROWS * K; idx += blockDim.x) {
         const int r = idx / K, i = idx % K;
-        hl_in[idx] = r < nr ? load_as_f32(in, (size_t)(row0 + r) * a.in_stride + a.in_off + (size_t)head * K + i, a.in_dtype) : 0.f;
+        hl_in[idx] = r < nr ? load_as_f32(in, (size_t)(row0 + r) * a.in_stride + a.in_off + in_head + i, a.in_dtype) : 0.f;
     }
     __syncthreads();
     const TW* w = (const TW*)a.weight;
     auto finish = [&](int r, int o, float acc) {
         const size_t row = row0 + r;
         if (a.gate_act) {
-            const float z = gate[row * a.gate_stride + a.gate_off + (size_t)head * N + o];
+            const float z = gate[row * a.gate_stride + a.gate_off + (a.gate_per_head ? (size_t)head : (size_t)head * N + o)];
             acc *= a.gate_act == 1 ? silu_f(z) : sigmoid_f(z);
         }
-        store_from_f32(out, row * a.out_stride + a.out_off + (size_t)head * N + o, a.out_dtype, acc);
+        store_from_f32(out, row * a.out_stride + a.out_off + out_head + o, a.out_dtype, acc);
     };
     if (a.transposed) {
         float* part = hl_in + HL_ROWS * K;
@@ -267,7 +269,8 @@ __global__ __launch_bounds__(256) void head_linear_mfma_kernel(picolm_head_linea
     const int n0 = (blockIdx.z * 4 + wave) * 32;
     if (n0 >= N) return;
     const int my_row = row0 + l32;
-    const size_t in_at = (size_t)min(my_row, n_rows - 1) * a.in_stride + a.in_off + (size_t)head * K + kq * 8;
+    const size_t in_at = (size_t)min(my_row, n_rows - 1) * a.in_stride + a.in_off + (size_t)head * (a.in_head_stride ? a.in_head_stride : K) + kq * 8;
+    const size_t out_head = (size_t)head * (a.out_head_stride ? a.out_head_stride : N);
     const bf16_t* w_row = (const bf16_t*)a.weight + ((size_t)head * N + min(n0 + l32, N - 1)) * K + kq * 8;
     f32x16 acc;
 #pragma unroll
@@ -294,10 +297,10 @@ __global__ __launch_bounds__(256) void head_linear_mfma_kernel(picolm_head_linea
         if (row >= (size_t)n_rows) continue;
         float y = acc[q];
         if (a.gate_act) {
-            const float z = gate[row * a.gate_stride + a.gate_off + (size_t)head * N + o];
+            const float z = gate[row * a.gate_stride + a.gate_off + (a.gate_per_head ? (size_t)head : (size_t)head * N + o)];
             y *= a.gate_act == 1 ? silu_f(z) : sigmoid_f(z);
         }
-        store_from_f32(out, row * a.out_stride + a.out_off + (size_t)head * N + o, a.out_dtype, y);
+        store_from_f32(out, row * a.out_stride + a.out_off + out_head + o, a.out_dtype, y);
     }
 }
 #define HL_MFMA_FROM_ROWS 32
@@ -309,12 +312,16 @@ extern "C" int picolm_call_head_linear(void* user, const picolm_step_view* v) {
     PICOLM_REQUIRE(a->heads > 0 && a->heads <= 65535 && a->in_dim > 0 && a->out_dim > 0 && known_dtype(a->weight_dt) && known_dtype(a->in_dtype) &&
                        known_dtype(a->out_dtype) && a->gate_act >= 0 && a->gate_act <= 2,
                    "head_linear: %d heads of %d to %d, or an unknown dtype or gate", a->heads, a->in_dim, a->out_dim);
-    PICOLM_REQUIRE(a->in_off >= 0 && a->in_off + (int64_t)a->heads * a->in_dim <= a->in_stride &&
+    const int64_t in_hs = a->in_head_stride ? a->in_head_stride : a->in_dim, out_hs = a->out_head_stride ? a->out_head_stride : a->out_dim;
+    PICOLM_REQUIRE(in_hs >= a->in_dim && out_hs >= a->out_dim, "head_linear: heads %lld and %lld apart overlap at sizes of %d and %d", (long long)in_hs,
+                   (long long)out_hs, a->in_dim, a->out_dim);
+    PICOLM_REQUIRE(a->in_off >= 0 && a->in_off + (a->heads - 1) * in_hs + a->in_dim <= a->in_stride &&
                        v->in_row_bytes >= (int64_t)a->in_stride * elem_bytes(a->in_dtype) && a->out_off >= 0 &&
-                       a->out_off + (int64_t)a->heads * a->out_dim <= a->out_stride &&
+                       a->out_off + (a->heads - 1) * out_hs + a->out_dim <= a->out_stride &&
                        v->out_row_bytes >= (int64_t)a->out_stride * elem_bytes(a->out_dtype),
                    "head_linear: rows too short for %d heads at the offsets named", a->heads);
-    PICOLM_REQUIRE(!a->gate_act || (v->extra[0] && a->gate_off >= 0 && a->gate_off + (int64_t)a->heads * a->out_dim <= a->gate_stride &&
+    PICOLM_REQUIRE(!a->gate_act || (v->extra[0] && a->gate_off >= 0 &&
+                                    a->gate_off + (int64_t)a->heads * (a->gate_per_head ? 1 : a->out_dim) <= a->gate_stride &&
                                     v->extra_row_bytes[0] >= (int64_t)a->gate_stride * 4),
                    "head_linear: the gate's rows of %d floats do not hold the heads at %d", a->gate_stride, a->gate_off);
     const size_t lds = sizeof(float) * (HL_ROWS * (size_t)a->in_dim + (a->transposed ? 4 * HL_ROWS * HL_COLS : 0));
@@ -322,7 +329,7 @@ extern "C" int picolm_call_head_linear(void* user, const picolm_step_view* v) {
                    a->in_dim, lds);
     if (v->rows <= 0) return 0;
     if (v->dtype == PICOLM_BF16 && a->weight_dt == PICOLM_BF16 && !a->transposed && v->rows >= HL_MFMA_FROM_ROWS && a->in_dim % 16 == 0 &&
-        a->in_off % 8 == 0 && a->in_stride % 8 == 0 && ceil_div(a->out_dim, 128) <= 65535) {
+        a->in_off % 8 == 0 && a->in_stride % 8 == 0 && in_hs % 8 == 0 && ceil_div(a->out_dim, 128) <= 65535) {
         head_linear_mfma_kernel<<<dim3(ceil_div(v->rows, 32), a->heads, ceil_div(a->out_dim, 128)), 256, 0, v->stream>>>(
             *a, v->in, v->out, (const float*)v->extra[0], v->rows);
         PICOLM_LAUNCH_CHECK("head_linear (matrix cores)");
@@ -414,5 +421,92 @@ extern "C" int picolm_call_forget_gates(void* user, const picolm_step_view* v) {
     forget_gates_kernel<<<blocks, 256, 0, v->stream>>>((const float*)v->in, a->in_stride, a->q_off, a->f_off, (float*)v->out, a->lower, a->bias,
                                                       a->channels, n);
     PICOLM_LAUNCH_CHECK("forget_gates");
+    return 0;
+}
+
+// ---- layer norm ---------------------------------------------------------------------------------------
+// One workgroup a row, two passes over the row in float: the mean, then the mean of the squared
+// deviations from it (not E[x^2] - mean^2, which loses the small variance of a row with a large mean).
+__global__ __launch_bounds__(1024) void layer_norm_kernel(const float* __restrict__ x, size_t x_stride, const int32_t* __restrict__ gather,
+                                                         void* __restrict__ out, size_t out_stride, int out_dt,
+                                                         const float* __restrict__ weight, const float* __restrict__ bias, int W, float eps) {
+    __shared__ float scratch[16];
+    const size_t row = blockIdx.x;
+    const float* xr = x + (gather ? (size_t)gather[row] : row) * x_stride;
+    float sum = 0.f;
+    for (int c = threadIdx.x; c < W; c += blockDim.x) sum += xr[c];
+    const float mean = block_sum(sum, scratch) / (float)W;
+    __syncthreads();                                   // (the scratch is read before it is written again)
+    float ssq = 0.f;
+    for (int c = threadIdx.x; c < W; c += blockDim.x) {
+        const float dev = xr[c] - mean;
+        ssq += dev * dev;
+    }
+    const float inv = 1.f / sqrtf(block_sum(ssq, scratch) / (float)W + eps);
+    for (int c = threadIdx.x; c < W; c += blockDim.x)
+        store_from_f32(out, row * out_stride + c, out_dt, (xr[c] - mean) * inv * weight[c] + (bias ? bias[c] : 0.f));
+}
+
+extern "C" int picolm_call_layer_norm(void* user, const picolm_step_view* v) {
+    const picolm_layer_norm_args* a = (const picolm_layer_norm_args*)user;
+    VIEW_REQUIRE("layer_norm", v);
+    PICOLM_REQUIRE(a && a->weight && v->in && v->out && v->in != v->out && a->width > 0 && known_dtype(a->out_dtype) && a->eps > 0.f,
+                   "layer_norm: weights or buffers are missing");
+    PICOLM_REQUIRE(v->in_row_bytes >= a->width * 4 && v->out_row_bytes >= a->width * elem_bytes(a->out_dtype),
+                   "layer_norm: rows too short for a width of %d", a->width);
+    PICOLM_REQUIRE(!a->gathers || v->want_rows, "layer_norm: the step names no wanted rows");
+    if (v->rows <= 0) return 0;
+    layer_norm_kernel<<<v->rows, a->width >= 2048 ? 1024 : 256, 0, v->stream>>>(
+        (const float*)v->in, (size_t)a->width, a->gathers ? v->want_rows : nullptr, v->out, (size_t)a->width, a->out_dtype, a->weight, a->bias,
+        a->width, a->eps);
+    PICOLM_LAUNCH_CHECK("layer_norm");
+    return 0;
+}
+
+// ---- rotation of stretches of a row by the token's position ---------------------------------------------
+// A thread a pair (or an entry that is only copied); a workgroup a row.
+__global__ void rotate_heads_kernel(picolm_rotate_heads_args a, const float* __restrict__ in, float* __restrict__ out,
+                                    const int32_t* __restrict__ tok_pos) {
+    const size_t row = blockIdx.x;
+    const int pairs = a.dims / 2, rest = a.width - a.dims, per_head = pairs + rest;
+    const int p = min(tok_pos[row], a.table_positions - 1);        // (the host has checked the step's positions against the table)
+    const float* cs = a.cos_table + (size_t)p * pairs;
+    const float* sn = a.sin_table + (size_t)p * pairs;
+    for (int idx = threadIdx.x; idx < a.heads * per_head; idx += blockDim.x) {
+        const int head = idx / per_head, j = idx % per_head;
+        const float* x = in + row * a.in_stride + a.in_off + (size_t)head * a.in_head_stride;
+        float* y = out + row * a.out_stride + a.out_off + (size_t)head * a.out_head_stride;
+        if (j < pairs) {
+            const int iu = a.half ? j : 2 * j, iv = a.half ? j + pairs : 2 * j + 1;
+            const float u = x[iu], w = x[iv], c = cs[j], s = sn[j];
+            y[iu] = u * c - w * s;
+            y[iv] = w * c + u * s;
+        } else {
+            y[a.dims + j - pairs] = x[a.dims + j - pairs];
+        }
+    }
+}
+
+extern "C" int picolm_call_rotate_heads(void* user, const picolm_step_view* v) {
+    const picolm_rotate_heads_args* a = (const picolm_rotate_heads_args*)user;
+    VIEW_REQUIRE("rotate_heads", v);
+    PICOLM_REQUIRE(a && a->cos_table && a->sin_table && v->in && v->out && v->tok_pos && v->rows == v->n_tokens,
+                   "rotate_heads: tables or buffers are missing (it covers the step's rows)");
+    PICOLM_REQUIRE(a->dims > 0 && a->dims % 2 == 0 && a->width >= a->dims && a->heads > 0 && a->table_positions > 0 &&
+                       a->in_head_stride >= (a->heads > 1 ? a->width : 0) && a->out_head_stride >= (a->heads > 1 ? a->width : 0),
+                   "rotate_heads: %d stretches of %d entries of which %d turn", a->heads, a->width, a->dims);
+    PICOLM_REQUIRE(a->in_off >= 0 && a->in_off + (int64_t)(a->heads - 1) * a->in_head_stride + a->width <= a->in_stride &&
+                       v->in_row_bytes >= (int64_t)a->in_stride * 4 && a->out_off >= 0 &&
+                       a->out_off + (int64_t)(a->heads - 1) * a->out_head_stride + a->width <= a->out_stride &&
+                       v->out_row_bytes >= (int64_t)a->out_stride * 4,
+                   "rotate_heads: rows too short for %d stretches at the offsets named", a->heads);
+    PICOLM_REQUIRE(v->in != v->out || (a->in_stride == a->out_stride && a->in_off == a->out_off && a->in_head_stride == a->out_head_stride),
+                   "rotate_heads: in place needs equal offsets and strides");
+    for (int i = 0; i < v->n_seq; ++i)
+        PICOLM_REQUIRE(v->recording || v->pos0[i] + v->n_new[i] <= a->table_positions,
+                       "rotate_heads: sequence %d reaches position %d, the tables hold %d", i, v->pos0[i] + v->n_new[i], a->table_positions);
+    if (v->rows <= 0) return 0;
+    rotate_heads_kernel<<<v->rows, 128, 0, v->stream>>>(*a, (const float*)v->in, (float*)v->out, v->tok_pos);
+    PICOLM_LAUNCH_CHECK("rotate_heads");
     return 0;
 }

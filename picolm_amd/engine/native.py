@@ -69,7 +69,7 @@ class _KVEntries:
             _raise(rc)
         G, d = spec.n_kv_heads, spec.head_dim
         self.spec = spec
-        self.ring_pages = min(window_ring_pages(spec.window), engine.info(5)) if spec.window > 0 else engine.info(5)
+        self.ring_pages = min(window_ring_pages(spec.window), engine.info(5)) if spec.window > 0 and not getattr(spec, "keeps_all", False) else engine.info(5)
         self.k = device_view(k.value, (spec.n_entries, n.value, G, kernels.PAGE_TOKENS, d), dtype, device, engine._handle)
         self.v = device_view(v.value, (spec.n_entries, n.value, G, spec.value_dim, kernels.PAGE_TOKENS), dtype, device, engine._handle)
 

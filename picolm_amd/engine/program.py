@@ -76,7 +76,7 @@ class Op(Structure):
 
 class KVGroup(Structure):
     _fields_ = [("n_entries", c_int32), ("n_kv_heads", c_int32), ("head_dim", c_int32), ("window", c_int32),
-                ("v_head_dim", c_int32)]
+                ("v_head_dim", c_int32), ("keeps_all", c_int32)]
 
 
 class StateGroup(Structure):
@@ -277,7 +277,7 @@ class BuiltProgram:
         self.failures = b.failures
         self.ops = (Op * len(b.ops))(*b.ops)
         self.buffers = (Buffer * len(b._specs))(*[Buffer(*s) for s in b._specs])
-        kv = [KVGroup(g.n_entries, g.n_kv_heads, g.head_dim, g.window, g.v_head_dim) for g in cache_spec.kv_groups]
+        kv = [KVGroup(g.n_entries, g.n_kv_heads, g.head_dim, g.window, g.v_head_dim, int(g.keeps_all)) for g in cache_spec.kv_groups]
         st = [StateGroup(g.n_entries, g.bytes_per_slot) for g in cache_spec.state_groups]
         self.kv_groups = (KVGroup * max(len(kv), 1))(*kv)
         self.state_groups = (StateGroup * max(len(st), 1))(*st)

@@ -75,11 +75,13 @@ class Workspace:
 @dataclass(frozen=True)
 class KVRequest:
     """A mixer's need for keys and values of each token.  `head_dim` is the size of a key;
-    `v_head_dim` that of a value where it differs (0: the same)."""
+    `v_head_dim` that of a value where it differs (0: the same).  `keeps_all` with a window: the
+    cache keeps every key (no ring of pages) and the window only bounds what a query visits."""
     n_kv_heads: int
     head_dim: int
     window: int = 0
     v_head_dim: int = 0
+    keeps_all: bool = False
 
     def __post_init__(self):
         if self.v_head_dim == self.head_dim:        # one way to say "the same": requests compare equal

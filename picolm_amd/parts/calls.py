@@ -16,7 +16,7 @@ class SinkAttentionArgs(Structure):
     _fields_ = [("n_heads", c_int32), ("n_kv_heads", c_int32), ("head_dim", c_int32), ("v_head_dim", c_int32),
                 ("in_stride", c_int32), ("q_off", c_int32), ("k_off", c_int32), ("v_off", c_int32), ("gate_off", c_int32),
                 ("scale", c_float), ("eps", c_float),
-                ("q_norm", c_void_p), ("k_norm", c_void_p), ("bias", c_void_p), ("bias_rows", c_int32), ("sink", c_void_p)]
+                ("q_norm", c_void_p), ("k_norm", c_void_p), ("bias", c_void_p), ("bias_rows", c_int32), ("sink", c_void_p), ("window", c_int32)]
 
 
 class ShortConvArgs(Structure):
@@ -56,7 +56,7 @@ class TokenShiftArgs(Structure):
 
 class GateRowsArgs(Structure):
     _fields_ = [("width", c_int32), ("act", c_int32), ("x_stride", c_int32), ("x_off", c_int32), ("x_dtype", c_int32),
-                ("g_stride", c_int32), ("g_off", c_int32), ("out_dtype", c_int32), ("bias", c_void_p)]
+                ("g_stride", c_int32), ("g_off", c_int32), ("out_dtype", c_int32), ("bias", c_void_p), ("g_per_row", c_int32)]
 
 
 class SliceNormArgs(Structure):
@@ -68,7 +68,8 @@ class HeadLinearArgs(Structure):
     _fields_ = [("weight", c_void_p), ("weight_dt", c_int32), ("heads", c_int32), ("in_dim", c_int32), ("out_dim", c_int32),
                 ("transposed", c_int32), ("in_stride", c_int32), ("in_off", c_int32), ("in_dtype", c_int32),
                 ("out_stride", c_int32), ("out_off", c_int32), ("out_dtype", c_int32),
-                ("gate_act", c_int32), ("gate_stride", c_int32), ("gate_off", c_int32)]
+                ("gate_act", c_int32), ("gate_stride", c_int32), ("gate_off", c_int32),
+                ("in_head_stride", c_int32), ("out_head_stride", c_int32), ("gate_per_head", c_int32)]
 
 
 class GatedPostnormArgs(Structure):
@@ -88,18 +89,31 @@ class DecayScanArgs(Structure):
 
 
 class RouteTopArgs(Structure):
-    _fields_ = [("bias", c_void_p), ("experts", c_int32), ("top", c_int32)]
+    _fields_ = [("bias", c_void_p), ("experts", c_int32), ("top", c_int32), ("scoring", c_int32), ("in_stride", c_int32),
+                ("scale", c_float)]
 
 
 class RoutedExpertsArgs(Structure):
     _fields_ = [("gate", c_void_p), ("up", c_void_p), ("down", c_void_p), ("weight_dt", c_int32), ("experts", c_int32),
-                ("top", c_int32), ("width", c_int32), ("ff", c_int32), ("adds", c_int32)]
+                ("top", c_int32), ("width", c_int32), ("ff", c_int32), ("adds", c_int32), ("identity", c_int32)]
+
+
+class LayerNormArgs(Structure):
+    _fields_ = [("weight", c_void_p), ("bias", c_void_p), ("width", c_int32), ("out_dtype", c_int32), ("eps", c_float),
+                ("gathers", c_int32)]
+
+
+class RotateHeadsArgs(Structure):
+    _fields_ = [("cos_table", c_void_p), ("sin_table", c_void_p), ("table_positions", c_int32), ("dims", c_int32), ("half", c_int32),
+                ("heads", c_int32), ("width", c_int32), ("in_stride", c_int32), ("in_off", c_int32), ("in_head_stride", c_int32),
+                ("out_stride", c_int32), ("out_off", c_int32), ("out_head_stride", c_int32)]
 
 
 GATE_NONE, GATE_SILU, GATE_SIGMOID = 0, 1, 2
 DECAY_PER_ROW, DECAY_EXPONENTIAL = 1, 2
 DECAY_SCAN_MAX_KEY_DIM = 256
-MAP_RELU_SQUARED, MAP_SOFTCAP = 1, 2
+MAP_RELU_SQUARED, MAP_SOFTCAP, MAP_SCALE = 1, 2, 3
+SCORE_PICKED_SOFTMAX, SCORE_SOFTMAX_ALL = 0, 1
 RULE_OUTER_PRODUCT, RULE_DELTA = 0, 1
 STATE_SCAN_MAX_KEY_DIM = 256
 SHORT_CONV_MAX_TAPS = 16

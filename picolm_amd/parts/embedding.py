@@ -79,10 +79,10 @@ class LMHead(Part):
     graph_safe = True      # launches depend on device memory only
 
     def __init__(self, name: str, vocab_size: int, hidden_size: int, embedding: TokenEmbedding, tied: bool,
-                 softcap: float = 0.0):
-        """`softcap` c > 0: logits <- c tanh(logits / c)."""
+                 softcap: float = 0.0, scale: float = 1.0):
+        """`scale`: the logits are multiplied by it; `softcap` c > 0: then logits <- c tanh(logits / c)."""
         self.name, self.V, self.D, self.embedding, self.tied = name, vocab_size, hidden_size, embedding, tied
-        self.softcap = float(softcap or 0.0)
+        self.softcap, self.scale = float(softcap or 0.0), float(scale)
         self.weight = None
 
     def tensor_specs(self):
@@ -104,6 +104,10 @@ class LMHead(Part):
             raise ValueError(f"head {self.name} has no weights loaded")
         logits = b.buffer("logits", self.V, torch.float32, ROWS_WANTED)
         b.linear(self.weight, src, logits, kernels.EPI_STORE, rows=ROWS_WANTED)
+        if self.scale != 1.0:
+            from .calls import MAP_SCALE, MapRowsArgs, emit_library_call
+            from ..engine.program import F32
+            emit_library_call(b, "map_rows", MapRowsArgs(MAP_SCALE, self.V, F32, F32, self.scale), logits, rows=ROWS_WANTED)
         if self.softcap > 0:
             from .calls import MAP_SOFTCAP, MapRowsArgs, emit_library_call
             from ..engine.program import F32
@@ -113,5 +117,7 @@ class LMHead(Part):
     def forward(self, h: torch.Tensor, logits: torch.Tensor) -> None:
         """The same on tensors, now."""
         kernels.gemm(h, self.weight, logits, kernels.EPI_STORE)
+        if self.scale != 1.0:
+            logits.mul_(self.scale)
         if self.softcap > 0:
             logits.copy_(self.softcap * torch.tanh(logits / self.softcap))

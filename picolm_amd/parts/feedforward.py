@@ -69,19 +69,35 @@ class ActivatedMLP(FeedForward):
 
 class RoutedExperts(FeedForward):
     """A feed-forward of many small gated experts of which every row uses a few:
-        z = W_router h + b;  the `top` largest z pick the experts (ties: the lower index);
-        w = softmax over the picked z alone;  out = sum_k w_k expert_k(h)  (+ shared(h))
-    expert(h) = down(silu(gate h) * (up h)), no biases; `shared_size` > 0 adds one more expert of
-    that inner width that every row passes.  The router's logits, the picks and their weights are
-    float; only the picked experts' weights are read."""
+        z = W_router h;  out = sum_k w_k expert_k(h)  (+ shared(h)) over the row's `top` picks k
+    scoring "picked_softmax": the largest z + b are picked (ties: the lower index) and w is the
+    softmax over the picked z + b alone.  scoring "softmax_all": s = softmax(z) over every router
+    output, the largest s + b are picked, and w = s_k / (sum of the picked s + 1e-20) * weight_scale.
+    expert(h) = down(silu(gate h) * (up h)), no biases; the last `identity` router outputs have no
+    tensors and stand for experts that give h back; `shared_size` > 0 adds one more expert of that
+    inner width that every row passes, multiplied by sigmoid(w_sg . h), one number a row, where
+    `shared_gate` names that vector's tensor.  `bias_name`: the tensor b, one entry per router
+    output.  The router's logits, the picks and their weights are float; only the picked experts'
+    weights are read."""
     graph_safe = True      # launches depend on device memory only
+    SCORINGS = {"picked_softmax": 0, "softmax_all": 1}
 
     def __init__(self, prefix: str, hidden_size: int, n_experts: int, top: int, expert_size: int, shared_size: int = 0,
-                 names=("gate", "up", "down")):
-        if not 1 <= top <= n_experts:
-            raise ValueError(f"{top} picks among {n_experts} experts")
+                 names=("gate", "up", "down"), scoring: str = "picked_softmax", identity: int = 0, weight_scale: float = 1.0,
+                 bias_name: str = "router.b", shared_gate: str | None = None):
+        if scoring not in self.SCORINGS:
+            raise ValueError(f"scoring '{scoring}': known are {', '.join(self.SCORINGS)}")
+        if n_experts < 1 or identity < 0 or not 1 <= top <= n_experts + identity:
+            raise ValueError(f"{top} picks among {n_experts} experts and {identity} that give their input back")
+        if shared_gate and not shared_size:
+            raise ValueError("a gate of the shared expert needs a shared expert")
         self.prefix, self.D, self.E, self.top, self.F, self.names = prefix, hidden_size, n_experts, top, expert_size, tuple(names)
-        self.router = Linear([prefix + "router"], [n_experts], hidden_size)
+        self.scoring, self.identity, self.weight_scale = scoring, int(identity), float(weight_scale)
+        self.bias_name, self.shared_gate = bias_name, shared_gate
+        self.outputs = n_experts + self.identity           # what the router gives a row
+        # the shared expert's gate is one more row of the router's product: both read h
+        self.router = Linear([prefix + "router"] + ([prefix + shared_gate] if shared_gate else []),
+                             [self.outputs] + ([1] if shared_gate else []), hidden_size)
         self.shared_gate_up = self.shared_down = None
         if shared_size:
             self.shared_gate_up = Linear([prefix + "shared." + names[0], prefix + "shared." + names[1]], [shared_size] * 2, hidden_size,
@@ -95,7 +111,7 @@ class RoutedExperts(FeedForward):
 
     def tensor_specs(self):
         from ..weights import TensorSpec
-        specs = [TensorSpec(self.prefix + "router.b", (self.E,), init="zeros")]
+        specs = [TensorSpec(self.prefix + self.bias_name, (self.outputs,), init="zeros")]
         for e in range(self.E):
             p = f"{self.prefix}e{e}."
             specs += [TensorSpec(p + self.names[0], (self.F, self.D)), TensorSpec(p + self.names[1], (self.F, self.D)),
@@ -111,29 +127,37 @@ class RoutedExperts(FeedForward):
                 ws = [w.to(torch.float32) for w in ws]
             return torch.stack(ws, dim=0).contiguous()
         self.gate, self.up, self.down = (stacked(n) for n in self.names)
-        self.router_bias = fetch.get(self.prefix + "router.b").to(torch.float32).contiguous()
+        self.router_bias = fetch.get(self.prefix + self.bias_name).to(torch.float32).contiguous()
 
     def emit(self, b, src, x: int, out_norm=None, out_norm_when: int = 0, accumulate: bool = True) -> None:
         """x (+)= the picked experts' weighted sum (+ the shared expert) for the rows h of `src`."""
         import torch
         from ..engine.program import _DT
-        from .calls import RoutedExpertsArgs, RouteTopArgs, emit_library_call
+        from .calls import GATE_SIGMOID, GateRowsArgs, RoutedExpertsArgs, RouteTopArgs, emit_library_call
         if self.gate is None:
             raise ValueError(f"the experts of {self.prefix} have no weights loaded")
         h = b.materialize(src)
-        logits = b.buffer("moe.logits", self.E, torch.float32)
+        n_logits = self.router.out_size
+        logits = b.buffer("moe.logits", n_logits, torch.float32)
         self.router.emit(b, h, logits, kernels.EPI_STORE)
         picks = b.buffer("moe.picks", 2 * self.top, torch.float32)
-        emit_library_call(b, "route_top", RouteTopArgs(b._ptr(self.router_bias), self.E, self.top), picks, inp=logits)
+        emit_library_call(b, "route_top", RouteTopArgs(b._ptr(self.router_bias), self.outputs, self.top, self.SCORINGS[self.scoring], n_logits,
+                                                       self.weight_scale), picks, inp=logits)
         written = accumulate
         if self.shared_size:
             act = b.buffer("ffn.act", self.shared_size, b.dtype)
             self.shared_gate_up.emit(b, h, act, kernels.EPI_SWIGLU)
+            if self.shared_gate:
+                # down(act) * s = down(act * s) for a number s a row: the hidden units take the gate
+                gated = b.buffer("ffn.act.gated", self.shared_size, b.dtype)
+                emit_library_call(b, "gate_rows", GateRowsArgs(self.shared_size, GATE_SIGMOID, self.shared_size, 0, _DT[b.dtype], n_logits,
+                                                               self.outputs, _DT[b.dtype], None, 1), gated, inp=act, extra=[logits])
+                act = gated
             self.shared_down.emit(b, act, x, kernels.EPI_ACCUMULATE if accumulate else kernels.EPI_STORE)
             written = True
         hidden = b.buffer("moe.hidden", self.top * self.F, torch.float32)
         args = RoutedExpertsArgs(b._ptr(self.gate), b._ptr(self.up), b._ptr(self.down), _DT[self.gate.dtype], self.E, self.top, self.D,
-                                 self.F, int(written))
+                                 self.F, int(written), self.identity)
         pair_out = b.buffer("moe.pairs", self.top * self.D, torch.float32)
         plan = b.buffer("moe.plan", self.top + self.E + 1, torch.float32)
         emit_library_call(b, "routed_experts", args, x, inp=h, extra=[picks, hidden, pair_out, plan])

@@ -50,3 +50,36 @@ class RMSNorm(Norm):
         out = ctx.ws.get(out_name, (n, self.size), ctx.dtype)
         kernels.rmsnorm(x, self.weight, self.eps, out, rows)
         return out
+
+
+class LayerNorm(Norm):
+    """out = (x - mean) / sqrt(var + eps) * w + b over a row, var the mean of the squared deviations
+    from the mean, in float; the bias is the tensor `<name>.b` (`bias=False`: none).  The products
+    around it cannot carry it as they carry an RMSNorm, so it is an operation of its own whose rows
+    the next product reads."""
+    graph_safe = True      # launches depend on device memory only
+
+    def __init__(self, name: str, size: int, eps: float, bias: bool = True):
+        self.name, self.size, self.eps, self.has_bias = name, size, float(eps), bool(bias)
+        self.weight = self.bias = None
+
+    def tensor_specs(self):
+        specs = [TensorSpec(self.name, (self.size,), init="ones")]
+        if self.has_bias:
+            specs.append(TensorSpec(self.name + ".b", (self.size,), init="zeros"))
+        return specs
+
+    def load(self, fetch, runtime: Runtime) -> None:
+        self.weight = fetch.get(self.name).to(torch.float32).contiguous()
+        self.bias = fetch.get(self.name + ".b").to(torch.float32).contiguous() if self.has_bias else None
+
+    def emit(self, b, x: int, rows: int = 0):
+        from ..engine.program import _DT, ROWS_WANTED, Rows
+        from .calls import LayerNormArgs, emit_library_call
+        if self.weight is None:
+            raise ValueError(f"norm {self.name} has no weights loaded")
+        wanted = rows == ROWS_WANTED
+        h = b.buffer("norm.final" if wanted else "norm.out", self.size, b.dtype, rows)
+        emit_library_call(b, "layer_norm", LayerNormArgs(b._ptr(self.weight), b._ptr(self.bias), self.size, _DT[b.dtype], self.eps,
+                                                        int(wanted)), h, inp=x, rows=rows)
+        return Rows(h)

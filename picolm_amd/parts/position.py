@@ -19,6 +19,8 @@ def rotary_inv_freq(head_dim: int, theta: float, scaling=None) -> torch.Tensor:
     inv = torch.pow(torch.tensor(float(theta), dtype=torch.float64), -2.0 * i / head_dim)
     if scaling is None:
         return inv
+    if hasattr(scaling, "fast"):
+        return _yarn_inv_freq(inv, head_dim, float(theta), scaling)
     factor, low, high = scaling.factor, scaling.low_freq_factor, scaling.high_freq_factor
     orig = float(scaling.original_max_position_embeddings)
     wavelen = 2.0 * math.pi / inv
@@ -26,6 +28,24 @@ def rotary_inv_freq(head_dim: int, theta: float, scaling=None) -> torch.Tensor:
     blended = (1.0 - smooth) * inv / factor + smooth * inv
     out = torch.where(wavelen > orig / low, inv / factor, blended)
     return torch.where(wavelen < orig / high, inv, out)
+
+
+def _yarn_inv_freq(inv: torch.Tensor, dims: int, theta: float, scaling) -> torch.Tensor:
+    """YaRN: pair i keeps its frequency below a first pair `lo`, has it divided by `factor` from a
+    last pair `hi` on, and a linear blend of the two between; lo and hi are the pairs that turn
+    `fast` and `slow` times within `original` positions (`scaling`: factor, original, fast, slow)."""
+    def pair_of(turns: float) -> float:
+        return dims * math.log(scaling.original / (2.0 * math.pi * turns)) / (2.0 * math.log(theta))
+    lo = max(math.floor(pair_of(scaling.fast)), 0)
+    hi = min(math.ceil(pair_of(scaling.slow)), dims - 1)
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    ramp = torch.clamp((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+    return inv / scaling.factor * ramp + inv * (1.0 - ramp)
+
+
+def rotary_magnitude(scaling) -> float:
+    """What cos and sin are multiplied by: 0.1 ln(factor) + 1 with YaRN scaling, 1 else."""
+    return 0.1 * math.log(scaling.factor) + 1.0 if scaling is not None and hasattr(scaling, "fast") else 1.0
 
 
 class RotaryEmbedding(PositionEncoding):
@@ -53,8 +73,9 @@ class RotaryEmbedding(PositionEncoding):
         ang = pos[:, None] * inv[None, :]                     # float32 product
         # cos/sin of the 32-bit angle, evaluated in float64 and rounded: correctly rounded
         # values, independent of the device's libm
-        self.cos = torch.cos(ang.double()).float().contiguous().to(runtime.device)
-        self.sin = torch.sin(ang.double()).float().contiguous().to(runtime.device)
+        mag = rotary_magnitude(self.scaling)
+        self.cos = (torch.cos(ang.double()) * mag).float().contiguous().to(runtime.device)
+        self.sin = (torch.sin(ang.double()) * mag).float().contiguous().to(runtime.device)
         self.n_positions = max_positions
 
     def rotary_tables(self):
