@@ -222,11 +222,63 @@ def _zarinex_pair(width: int, heads: int, kv_rank: int, experts: int, top: int, 
     return zar, beg
 
 
+def _satedra_pair(width: int, heads: int, kv_rank: int, rot_dim: int, window: int, experts: int, top: int, vocab: int, runs: int):
+    """A Satedra of `runs` layers with query heads of 128 (of which `rot_dim` entries turn), values of
+    128 read out of latents of `kv_rank`, every second layer reading the latents of the one before it,
+    windows of `window` keys in the layers that keep latents and of half as many in those that read
+    them, `experts` experts as wide as the model of which a token uses `top` (two more router outputs
+    give the input back) beside a shared one; and the Zarinex of as many latent-attention layers of the
+    same width, heads, vocabulary, experts and a cached key as long (kv_rank + rot_dim)."""
+    scaling = dict(factor=8.0, original=4096, fast=32.0, slow=1.0)
+    mlp = dict(kind="moe", router=dict(experts=experts, top=top, identity=2, scale=1.0), expert=dict(ff=width), shared=dict(ff=width))
+    layers = []
+    for i in range(runs):
+        m = dict(heads=heads, dim=128 - rot_dim, rot_dim=rot_dim, vdim=128, kv_rank=kv_rank, scale=128 ** -0.5,
+                 mask=dict(size=window if i % 2 == 0 else max(window // 2, 1)), rot=dict(base=10000.0, dims=rot_dim, scaling=scaling))
+        if i % 2:
+            m["kv_from"] = i - 1
+        layers.append(dict(type="latent_attention", mixer=m, mlp=mlp))
+    sat = dict(architecture="Satedra", vocab=vocab, width=width, norm=dict(eps=1e-6), logit_scale=1.0, layers=layers)
+    key = kv_rank + rot_dim
+    zmlp = dict(kind="moe", router=dict(experts=experts, top=top), expert=dict(ff=width), shared=dict(ff=width))
+    zar = dict(architecture="Zarinex", vocab=vocab, width=width, norm=dict(eps=1e-6), postln_alpha=1.0,
+               layers=[dict(type="latent_attention", mixer=dict(heads=heads, dim=128, vdim=128, kv_rank=key, q_rank=3 * key, scale=128 ** -0.5),
+                            mlp=zmlp) for _ in range(runs)])
+    return sat, zar
+
+
+def _satedra_rooflines(cfg: dict, T: int, n_seq: int, context: int) -> dict:
+    """As _zarinex_rooflines: the attention over the keys a window lets a query see, [latent | rotated
+    part] as the key and the latent as the value, at the bf16 matrix peak; the picked experts' products
+    at the bf16 matrix peak (every pick counted as a real expert); in a decode step a window's keys
+    and values once per sequence and the weights of the experts that the step's tokens can pick at
+    most, at HBM's peak."""
+    mfma, hbm = PEAK_TFLOPS["bf16"] * 1e12, HBM_PEAK_GBS * 1e9
+    names = ("sink_attention", "routed_experts")
+    pre, dec = {k: 0.0 for k in names}, {k: 0.0 for k in names}
+    D = cfg["width"]
+    for layer in cfg["layers"]:
+        m = layer["mixer"]
+        window = (m.get("mask") or {}).get("size", 0) or T + context
+        seen = sum(min(i + 1, window) for i in range(T))
+        pre["sink_attention"] += 2.0 * m["heads"] * (2 * m["kv_rank"] + m["rot_dim"]) * seen / mfma
+        dec["sink_attention"] += n_seq * min(context, window) * (2 * m["kv_rank"] + m["rot_dim"]) * 2 / hbm
+        mlp = layer.get("mlp")
+        if mlp and mlp["kind"] == "moe":
+            E, top, F = mlp["router"]["experts"], mlp["router"]["top"], mlp["expert"]["ff"]
+            pre["routed_experts"] += 2.0 * 3 * T * top * D * F / mfma
+            dec["routed_experts"] += min(n_seq * top, E) * 3 * D * F * 2 / hbm
+    return {"prefill": pre, "decode": dec}
+
+
 DESIGN_SIZES = {
     "begopel": [("width 1024", (1024, 8, 2, 4096, 32000, 2, 2)), ("width 2048", (2048, 16, 4, 8192, 32000, 2, 0)),
                 ("width 4096", (4096, 32, 8, 14336, 128256, 1, 0))],
     "zarinex": [("width 1024", (1024, 8, 128, 8, 2, 32000, 4)), ("width 2048", (2048, 16, 128, 8, 2, 32000, 4)),
                 ("width 4096", (4096, 32, 128, 16, 2, 128256, 2)), ("width 4096, latents of 512", (4096, 32, 512, 16, 2, 128256, 2))],
+    "satedra": [("width 1024", (1024, 8, 96, 32, 1024, 8, 2, 32000, 4)), ("width 2048", (2048, 16, 96, 32, 1024, 8, 2, 32000, 4)),
+                ("width 4096", (4096, 32, 96, 32, 4096, 16, 2, 128256, 2)),
+                ("width 4096, latents of 512", (4096, 32, 512, 64, 4096, 16, 2, 128256, 2))],
 }
 
 
@@ -263,7 +315,7 @@ def _zarinex_rooflines(cfg: dict, T: int, n_seq: int, context: int) -> dict:
 def design_comparison(design: str, T: int, n_seq: int, context: int, steps: int) -> dict:
     """Prefill and decode throughput of `design` at a few sizes that resemble real layers (random
     weights), beside the closest model the library has at equal size (for Begopel the Llama, for
-    Zarinex the Begopel), and the GPU time of one prefill step and one decode step by operation."""
+    Zarinex the Begopel, for Satedra the Zarinex), and the GPU time of one prefill step and one decode step by operation."""
     import torch
 
     from picolm_amd.config import LlamaConfig, resolve
@@ -323,6 +375,14 @@ def design_comparison(design: str, T: int, n_seq: int, context: int, steps: int)
 
     for name, size in DESIGN_SIZES[design]:
         print(f"[bench] {design} {name}", file=sys.stderr, flush=True)
+        if design == "satedra":
+            sat, zar = _satedra_pair(*size)
+            a = measure(resolve(sat).parse_config(sat), sat["vocab"])
+            b = measure(resolve(zar).parse_config(zar), zar["vocab"])
+            out["sizes"].append({"size": name, "layer_runs": len(sat["layers"]), design: a, "zarinex": b,
+                                 "fraction_of_roofline": fractions_of(_satedra_rooflines(sat, T, n_seq, context), a),
+                                 "zarinex_fraction_of_roofline": fractions_of(_zarinex_rooflines(zar, T, n_seq, context), b)})
+            continue
         if design == "zarinex":
             zar, beg = _zarinex_pair(*size)
             a = measure(resolve(zar).parse_config(zar), zar["vocab"])
@@ -378,7 +438,7 @@ def main() -> int:
                          "read on the host; 0: the host reads every step's tokens first")
     ap.add_argument("--design", choices=sorted(DESIGN_SIZES), default="",
                     help="instead of the record: prefill and decode throughput of another design at a few sizes beside the "
-                         "Llama of equal size, with the GPU time of a step by operation, as one JSON line")
+                         "closest model of equal size, with the GPU time of a step by operation, as one JSON line")
     args = ap.parse_args()
     if args.design:
         print(json.dumps(design_comparison(args.design, args.prefill_tokens, args.batch or 8, 1024, args.steps or 32)))

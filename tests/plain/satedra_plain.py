@@ -79,7 +79,7 @@ def latent_keys(h, W, p, m, eps, positions):
 
 
 def latent_attention(h, W, p, m, eps, kv, positions=None):
-    """m: {heads, dim, rot_dim, vdim, kv_rank, scale, mask: {size}, rot}; kv = (c, k_rot) of this layer
+    """m: {heads, dim, rot_dim, vdim, kv_rank, scale, mask: {size} (or none), rot}; kv = (c, k_rot) of this layer
     or of the one it reads."""
     H, d, dr, dv = m["heads"], m["dim"], m["rot_dim"], m["vdim"]
     T = h.shape[0]
@@ -89,7 +89,7 @@ def latent_attention(h, W, p, m, eps, kv, positions=None):
     q_plain, q_rot = q[..., :d], rotate(q[..., d:], positions, m["rot"])
     k = (c @ W[p + "uk"].T).reshape(T, H, d)
     v = (c @ W[p + "uv"].T).reshape(T, H, dv)
-    window = m["mask"]["size"]
+    window = (m.get("mask") or {}).get("size") or T           # no mask: every earlier key
     out = np.zeros((T, H, dv))
     for i in range(T):
         lo = max(0, i - window + 1)
