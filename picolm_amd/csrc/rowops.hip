@@ -180,10 +180,10 @@ extern "C" int picolm_call_slice_norm(void* user, const picolm_step_view* v) {
 #define HL_COLS 64
 template <typename TW>
 __global__ __launch_bounds__(256) void head_linear_kernel(picolm_head_linear_args a, const void* __restrict__ in, void* __restrict__ out,
-                                                          const float* __restrict__ gate, int n_rows) {
+                                                          const float* __restrict__ gate, int n_rows, int cols) {
     extern __shared__ float hl_in[];      // [HL_ROWS][in_dim] | partial sums [4][HL_ROWS][HL_COLS] (transposed)
     const int head = blockIdx.y, row0 = blockIdx.x * HL_ROWS, nr = min(HL_ROWS, n_rows - row0);
-    const int K = a.in_dim, N = a.out_dim, o0 = blockIdx.z * HL_COLS;
+    const int K = a.in_dim, N = a.out_dim, o0 = blockIdx.z * cols;       // (cols is HL_COLS when transposed)
     const size_t in_head = (size_t)head * (a.in_head_stride ? a.in_head_stride : K), out_head = (size_t)head * (a.out_head_stride ? a.out_head_stride : N);
     for (int idx = threadIdx.x; idx < HL_ROWS * K; idx += blockDim.x) {
         const int r = idx / K, i = idx % K;
@@ -227,7 +227,7 @@ __global__ __launch_bounds__(256) void head_linear_kernel(picolm_head_linear_arg
     } else {
         const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
         const TW* wh = w + (size_t)head * N * K;
-        const int o_end = min(N, o0 + HL_COLS);
+        const int o_end = min(N, o0 + cols);
         for (int ob = o0 + wave * 4; ob < o_end; ob += 16) {        // four waves, four outputs each at a time
             float acc[4][HL_ROWS];
 #pragma unroll
@@ -335,11 +335,15 @@ extern "C" int picolm_call_head_linear(void* user, const picolm_step_view* v) {
         PICOLM_LAUNCH_CHECK("head_linear (matrix cores)");
         return 0;
     }
-    const dim3 grid(ceil_div(v->rows, HL_ROWS), a->heads, ceil_div(a->out_dim, HL_COLS));
+    // a step of few rows has few workgroups, each with a chain of loads and sums in a row: not transposed, a workgroup
+    // then takes 16 outputs (its four waves four each, once) instead of 64
+    const int row_groups = ceil_div(v->rows, HL_ROWS);
+    const int cols = !a->transposed && (int64_t)row_groups * a->heads * ceil_div(a->out_dim, HL_COLS) < 256 && ceil_div(a->out_dim, 16) <= 65535 ? 16 : HL_COLS;
+    const dim3 grid(row_groups, a->heads, ceil_div(a->out_dim, cols));
     if (a->weight_dt == PICOLM_F32)
-        head_linear_kernel<float><<<grid, 256, lds, v->stream>>>(*a, v->in, v->out, (const float*)v->extra[0], v->rows);
+        head_linear_kernel<float><<<grid, 256, lds, v->stream>>>(*a, v->in, v->out, (const float*)v->extra[0], v->rows, cols);
     else
-        head_linear_kernel<bf16_t><<<grid, 256, lds, v->stream>>>(*a, v->in, v->out, (const float*)v->extra[0], v->rows);
+        head_linear_kernel<bf16_t><<<grid, 256, lds, v->stream>>>(*a, v->in, v->out, (const float*)v->extra[0], v->rows, cols);
     PICOLM_LAUNCH_CHECK("head_linear");
     return 0;
 }
