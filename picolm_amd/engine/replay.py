@@ -17,11 +17,15 @@ import sys
 import numpy as np
 
 from .builder import load_model
-from .session import Session
+from .session import PAGE_TOKENS, Session
 
 
 class TraceError(ValueError):
     pass
+
+
+# --max-tokens counts tokens, the cache counts pages, and every live request's last page is partly empty
+PADDED_REQUESTS = 256
 
 
 class Replayer:
@@ -74,10 +78,11 @@ def main(argv=None) -> int:
     ap.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
     ap.add_argument("--out", required=True, help="folder for <step>.f32 files")
     ap.add_argument("--max-tokens", type=int, required=True,
-                    help="most tokens live requests hold together, each rounded up to 64")
+                    help="most tokens live requests hold together (the cache rounds each request up to a page of 64; "
+                         f"room for that rounding of up to {PADDED_REQUESTS} live requests is added)")
     args = ap.parse_args(argv)
     model = load_model(args.model, dtype=args.dtype)
-    session = Session(model, max_tokens=args.max_tokens)
+    session = Session(model, max_tokens=args.max_tokens + PADDED_REQUESTS * PAGE_TOKENS)
     rp = Replayer(session, args.out)
     for line in sys.stdin:
         line = line.strip()

@@ -507,3 +507,21 @@ def test_trace_replay_and_command_line(folder_a, tmp_path):
     assert r.returncode == 0, r.stderr
     assert len(r.stdout.split()) == 4
     assert int(r.stdout.split()[0]) == int(np.argmax(tb.logits[-1]))
+
+
+def test_trace_replay_counts_tokens_where_the_cache_counts_pages(folder_a, tmp_path):
+    """--max-tokens is the sum of the live requests' tokens; each of them fills its last page only partly."""
+    cfg = st.CONFIGS["A"]
+    seqs = {f"r{i}": tokens_for(cfg, 3 + i, 80 + i) for i in range(6)}
+    steps = [{"step": 0, "entries": [{"id": k, "tokens": q[:-1], "want": [len(q) - 2]} for k, q in seqs.items()], "end": []},
+             {"step": 1, "entries": [{"id": k, "tokens": q[-1:], "want": [0]} for k, q in seqs.items()], "end": list(seqs)}]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = str(tmp_path / "out")
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder_a, "--dtype", "float32", "--out", out,
+                        "--max-tokens", str(sum(len(q) for q in seqs.values()))], input="\n".join(json.dumps(s) for s in steps) + "\n",
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr
+    got = [np.fromfile(os.path.join(out, f"{i}.f32"), dtype="<f4").reshape(-1, cfg["vocab"]) for i in (0, 1)]
+    for row, q in enumerate(seqs.values()):
+        t = truth_of("A", 0, q)
+        assert st.near(got[0][row], t, len(q) - 2, "float32") and st.near(got[1][row], t, len(q) - 1, "float32")
