@@ -217,6 +217,12 @@ def test_a_batch_of_unequal_requests_equals_each_alone(which, dtype):
     for i, n in enumerate(lens):
         assert st.near(got[at:at + n], truth[i], slice(0, n), dtype), ("prompt", i)
         at += n
+    # and against each alone, much closer than the plain model is in bfloat16: what else is in the batch does not show
+    alone = new_session(model, 512)
+    at = 0
+    for i, n in enumerate(lens):
+        assert st.distance(got[at:at + n], run_whole(alone, seqs[i][:n])) <= (1e-5 if dtype == "float32" else 0.03), ("alone", i)
+        at += n
     # the shorter ones end earlier: after two steps the first two leave the batch
     live = list(range(len(seqs)))
     for j in range(n_dec):
