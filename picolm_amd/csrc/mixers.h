@@ -252,12 +252,21 @@ int picolm_call_layer_norm(void* user, const picolm_step_view* v);
 //   in: float rows [in_stride], stretch h at in_off + h in_head_stride; out: float rows
 //   [out_stride], stretch h at out_off + h out_head_stride (in place: out names the same buffer,
 //   and the offsets and strides are equal).
+// In the same pass, where in and out are two buffers: `more_heads` further stretches of the same
+// shape at offsets and strides of their own (a key part beside the queries' heads, say), and a
+// stretch of `norm_width` columns at norm_in_off that is divided by its root mean square (eps inside
+// the root), multiplied by norm_weight and written at norm_out_off (more_heads = 0, norm_weight
+// null: none).
 typedef struct {
     const float* cos_table;  // [table_positions][dims / 2]
     const float* sin_table;
     int32_t table_positions, dims, half, heads, width;      // width: entries of a stretch, >= dims
     int32_t in_stride, in_off, in_head_stride;
     int32_t out_stride, out_off, out_head_stride;
+    int32_t more_heads, more_in_off, more_in_head_stride, more_out_off, more_out_head_stride;
+    const float* norm_weight;  // [norm_width] or null
+    int32_t norm_width, norm_in_off, norm_out_off;
+    float norm_eps;
 } picolm_rotate_heads_args;
 int picolm_call_rotate_heads(void* user, const picolm_step_view* v);
 

@@ -468,18 +468,23 @@ extern "C" int picolm_call_layer_norm(void* user, const picolm_step_view* v) {
 }
 
 // ---- rotation of stretches of a row by the token's position ---------------------------------------------
-// A thread a pair (or an entry that is only copied); a workgroup a row.
-__global__ void rotate_heads_kernel(picolm_rotate_heads_args a, const float* __restrict__ in, float* __restrict__ out,
-                                    const int32_t* __restrict__ tok_pos) {
+// A thread a pair (or an entry that is only copied); a workgroup a row.  The stretches of the second group follow
+// those of the first in the threads' order; the normed stretch comes last and takes the whole workgroup's sum.
+__global__ __launch_bounds__(256) void rotate_heads_kernel(picolm_rotate_heads_args a, const float* __restrict__ in, float* __restrict__ out,
+                                                           const int32_t* __restrict__ tok_pos) {
+    __shared__ float scratch[16];
     const size_t row = blockIdx.x;
     const int pairs = a.dims / 2, rest = a.width - a.dims, per_head = pairs + rest;
     const int p = min(tok_pos[row], a.table_positions - 1);        // (the host has checked the step's positions against the table)
     const float* cs = a.cos_table + (size_t)p * pairs;
     const float* sn = a.sin_table + (size_t)p * pairs;
-    for (int idx = threadIdx.x; idx < a.heads * per_head; idx += blockDim.x) {
+    for (int idx = threadIdx.x; idx < (a.heads + a.more_heads) * per_head; idx += blockDim.x) {
         const int head = idx / per_head, j = idx % per_head;
-        const float* x = in + row * a.in_stride + a.in_off + (size_t)head * a.in_head_stride;
-        float* y = out + row * a.out_stride + a.out_off + (size_t)head * a.out_head_stride;
+        const bool first = head < a.heads;
+        const float* x = in + row * a.in_stride + (first ? a.in_off + (size_t)head * a.in_head_stride
+                                                         : a.more_in_off + (size_t)(head - a.heads) * a.more_in_head_stride);
+        float* y = out + row * a.out_stride + (first ? a.out_off + (size_t)head * a.out_head_stride
+                                                     : a.more_out_off + (size_t)(head - a.heads) * a.more_out_head_stride);
         if (j < pairs) {
             const int iu = a.half ? j : 2 * j, iv = a.half ? j + pairs : 2 * j + 1;
             const float u = x[iu], w = x[iv], c = cs[j], s = sn[j];
@@ -489,6 +494,13 @@ __global__ void rotate_heads_kernel(picolm_rotate_heads_args a, const float* __r
             y[a.dims + j - pairs] = x[a.dims + j - pairs];
         }
     }
+    if (!a.norm_weight) return;                    // (the same for every thread of the grid)
+    const float* xr = in + row * a.in_stride + a.norm_in_off;
+    float ssq = 0.f;
+    for (int c = threadIdx.x; c < a.norm_width; c += blockDim.x) ssq += xr[c] * xr[c];
+    ssq = block_sum(ssq, scratch);
+    const float inv = 1.f / sqrtf(ssq / (float)a.norm_width + a.norm_eps);
+    for (int c = threadIdx.x; c < a.norm_width; c += blockDim.x) out[row * a.out_stride + a.norm_out_off + c] = xr[c] * inv * a.norm_weight[c];
 }
 
 extern "C" int picolm_call_rotate_heads(void* user, const picolm_step_view* v) {
@@ -504,13 +516,24 @@ extern "C" int picolm_call_rotate_heads(void* user, const picolm_step_view* v) {
                        a->out_off + (int64_t)(a->heads - 1) * a->out_head_stride + a->width <= a->out_stride &&
                        v->out_row_bytes >= (int64_t)a->out_stride * 4,
                    "rotate_heads: rows too short for %d stretches at the offsets named", a->heads);
-    PICOLM_REQUIRE(v->in != v->out || (a->in_stride == a->out_stride && a->in_off == a->out_off && a->in_head_stride == a->out_head_stride),
-                   "rotate_heads: in place needs equal offsets and strides");
+    PICOLM_REQUIRE(v->in != v->out || (a->in_stride == a->out_stride && a->in_off == a->out_off && a->in_head_stride == a->out_head_stride &&
+                                       !a->more_heads && !a->norm_weight),
+                   "rotate_heads: in place needs equal offsets and strides, and no further stretches");
+    PICOLM_REQUIRE(a->more_heads >= 0 && (!a->more_heads ||
+                                          (a->more_in_head_stride >= (a->more_heads > 1 ? a->width : 0) &&
+                                           a->more_out_head_stride >= (a->more_heads > 1 ? a->width : 0) && a->more_in_off >= 0 &&
+                                           a->more_in_off + (int64_t)(a->more_heads - 1) * a->more_in_head_stride + a->width <= a->in_stride &&
+                                           a->more_out_off >= 0 &&
+                                           a->more_out_off + (int64_t)(a->more_heads - 1) * a->more_out_head_stride + a->width <= a->out_stride)),
+                   "rotate_heads: rows too short for %d further stretches at the offsets named", a->more_heads);
+    PICOLM_REQUIRE(!a->norm_weight || (a->norm_width > 0 && a->norm_eps > 0.f && a->norm_in_off >= 0 && a->norm_in_off + a->norm_width <= a->in_stride &&
+                                       a->norm_out_off >= 0 && a->norm_out_off + a->norm_width <= a->out_stride),
+                   "rotate_heads: rows too short for a normed stretch of %d columns at the offsets named", a->norm_width);
     for (int i = 0; i < v->n_seq; ++i)
         PICOLM_REQUIRE(v->recording || v->pos0[i] + v->n_new[i] <= a->table_positions,
                        "rotate_heads: sequence %d reaches position %d, the tables hold %d", i, v->pos0[i] + v->n_new[i], a->table_positions);
     if (v->rows <= 0) return 0;
-    rotate_heads_kernel<<<v->rows, 128, 0, v->stream>>>(*a, (const float*)v->in, (float*)v->out, v->tok_pos);
+    rotate_heads_kernel<<<v->rows, 256, 0, v->stream>>>(*a, (const float*)v->in, (float*)v->out, v->tok_pos);
     PICOLM_LAUNCH_CHECK("rotate_heads");
     return 0;
 }

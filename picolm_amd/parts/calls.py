@@ -106,7 +106,10 @@ class LayerNormArgs(Structure):
 class RotateHeadsArgs(Structure):
     _fields_ = [("cos_table", c_void_p), ("sin_table", c_void_p), ("table_positions", c_int32), ("dims", c_int32), ("half", c_int32),
                 ("heads", c_int32), ("width", c_int32), ("in_stride", c_int32), ("in_off", c_int32), ("in_head_stride", c_int32),
-                ("out_stride", c_int32), ("out_off", c_int32), ("out_head_stride", c_int32)]
+                ("out_stride", c_int32), ("out_off", c_int32), ("out_head_stride", c_int32),
+                ("more_heads", c_int32), ("more_in_off", c_int32), ("more_in_head_stride", c_int32), ("more_out_off", c_int32),
+                ("more_out_head_stride", c_int32), ("norm_weight", c_void_p), ("norm_width", c_int32), ("norm_in_off", c_int32),
+                ("norm_out_off", c_int32), ("norm_eps", c_float)]
 
 
 GATE_NONE, GATE_SILU, GATE_SIGMOID = 0, 1, 2

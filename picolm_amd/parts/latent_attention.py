@@ -183,13 +183,11 @@ class RotatedLatentAttention(Mixer):
         weight_dt = _DT[self.uk.dtype]
         emit_library_call(b, "head_linear", HeadLinearArgs(b._ptr(self.uk), weight_dt, H, d, r, 0 if self.uk_transposed else 1, width, 0, F32,
                                                            q_wide + key, 0, F32, GATE_NONE, 0, 0, d + dr, key, 0), qc, inp=rows)
-        turn = lambda heads, in_off, in_hs, out_off, out_hs: emit_library_call(
-            b, "rotate_heads", RotateHeadsArgs(b._ptr(cos), b._ptr(sin), cos.shape[0], dr, style, heads, dr, width, in_off, in_hs,
-                                               q_wide + key, out_off, out_hs), qc, inp=rows)
-        turn(H, d, d + dr, r, key)
-        if not self.reads_latents:
-            emit_library_call(b, "slice_norm", SliceNormArgs(b._ptr(self.c_norm), r, width, c_at, q_wide + key, q_wide, F32, self.eps), qc, inp=rows)
-            turn(1, c_at + r, 0, q_wide + r, 0)
+        # one pass over a token's row: the queries' rotated parts behind each head's W_uk^T q, and for a layer with latents of its own
+        # the normed latent and the rotated key part behind the queries
+        own = (1, c_at + r, 0, q_wide + r, 0, b._ptr(self.c_norm), r, c_at, q_wide, self.eps) if not self.reads_latents else ()
+        emit_library_call(b, "rotate_heads", RotateHeadsArgs(b._ptr(cos), b._ptr(sin), cos.shape[0], dr, style, H, dr, width, d, d + dr,
+                                                             q_wide + key, r, key, *own), qc, inp=rows)
         scratch = b.buffer("rla.q.rows", q_wide, b.dtype)
         att = b.buffer("rla.att", H * r, b.dtype)
         args = SinkAttentionArgs(H, 1, key, r, q_wide + key, 0, q_wide, q_wide, -1, self.scale, self.eps, None, None, None, 0, None,
