@@ -79,10 +79,13 @@ def main(argv=None) -> int:
     ap.add_argument("--out", required=True, help="folder for <step>.f32 files")
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold together (the cache rounds each request up to a page of 64; "
-                         f"room for that rounding of up to {PADDED_REQUESTS} live requests is added)")
+                         "room for that rounding is added, see --live-requests)")
+    ap.add_argument("--live-requests", type=int, default=PADDED_REQUESTS,
+                    help="the most requests live at a time: the cache gets a page for each beside the token budget "
+                         f"(default {PADDED_REQUESTS})")
     args = ap.parse_args(argv)
     model = load_model(args.model, dtype=args.dtype)
-    session = Session(model, max_tokens=args.max_tokens + PADDED_REQUESTS * PAGE_TOKENS)
+    session = Session(model, max_tokens=args.max_tokens + max(args.live_requests, 0) * PAGE_TOKENS)
     rp = Replayer(session, args.out)
     for line in sys.stdin:
         line = line.strip()

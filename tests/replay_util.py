@@ -13,11 +13,11 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 class TraceRun:
-    def __init__(self, model_dir, dtype, out_dir, max_tokens, env=None):
+    def __init__(self, model_dir, dtype, out_dir, max_tokens, env=None, more=()):
         self.out_dir = out_dir
         self.proc = subprocess.Popen(
             [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model_dir, "--dtype", dtype,
-             "--out", out_dir, "--max-tokens", str(max_tokens)],
+             "--out", out_dir, "--max-tokens", str(max_tokens), *more],
             stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True, bufsize=1, env=env)
         self.n = 0
 

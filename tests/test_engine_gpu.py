@@ -50,7 +50,7 @@ def requests_and_truth(folders):
 def test_replay_whole_tail_and_batches(which, dtype, folders, requests_and_truth, tmp_path):
     reqs, truth = requests_and_truth[which]
     one_batch = sum((len(r) + 63) // 64 for r in reqs[3:]) * 64          # room for the larger batch only
-    tr = TraceRun(folders[which], dtype, str(tmp_path / "out"), one_batch)
+    tr = TraceRun(folders[which], dtype, str(tmp_path / "out"), one_batch, more=("--live-requests", "0"))
     worst = 0.0
 
     def check(got, ref, what):
@@ -92,7 +92,7 @@ def test_replay_whole_tail_and_batches(which, dtype, folders, requests_and_truth
 
 
 def test_replay_reports_a_full_cache(folders, tmp_path):
-    tr = TraceRun(folders["A"], "float32", str(tmp_path / "o"), 64)
+    tr = TraceRun(folders["A"], "float32", str(tmp_path / "o"), 64, more=("--live-requests", "0"))      # one page and no more
     assert tr.step([("a", [1] * 60, [59])]).shape == (1, 256)
     with pytest.raises(RuntimeError):
         tr.step([("b", [1] * 10, [0])])          # no page left: the program stops with an error
