@@ -51,7 +51,7 @@ def _load_builtin() -> None:
     global _BUILTIN_LOADED
     if not _BUILTIN_LOADED:
         _BUILTIN_LOADED = True
-        from ..engine import begopel, llama, satedra, zarinex  # noqa: F401
+        from ..engine import begopel, kekelix, llama, satedra, zarinex  # noqa: F401
 
 
 _OUTSIDE_LOADED = False

@@ -114,7 +114,9 @@ int picolm_kv_page_order(int dt, int d, int32_t* k_idx, int32_t* v_idx);
 // of the softmax's denominator and adds nothing to the numerator), and a gate (the output of head h is
 // multiplied by sigmoid(gate[token * gate_stride + h * v_head_dim + c]), float rows), and a window
 // of the operation's own (mask_window > 0: a query sees that many keys, no more than the `window`
-// that the pages and the decode step's work list are laid out for; zero: `window` itself).
+// that the pages and the decode step's work list are laid out for; zero: `window` itself), a stretch
+// (mask_chunk > 0: a query sees only the keys of its own stretch of that many positions, counted from
+// the sequence's first, up to itself), and float output rows whatever the dtype (out_float = 1).
 typedef struct {
     int32_t v_head_dim;
     const float* bias;
@@ -123,6 +125,8 @@ typedef struct {
     const float* gate;
     int32_t gate_stride;
     int32_t mask_window;
+    int32_t mask_chunk;
+    int32_t out_float;
 } picolm_attn_extras;
 // picolm_attn_prefill_generic / picolm_attn_decode_generic over pages kept as plain arrays K[64][d],
 // V^T[dv][64] whatever the dtype and head size, with the extras above; out rows are [H][dv] and the

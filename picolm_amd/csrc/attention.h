@@ -56,10 +56,22 @@ struct AttnArgs {
     // and the decode step's work list are laid out for (several layers with windows of their own
     // may read one entry); zero: `window` itself
     int mask_window;
+    // a query sees only the keys of its own stretch of `mask_chunk` positions (stretches are counted
+    // from position 0 of the sequence) up to itself; zero: no such bound
+    int mask_chunk;
+    // the output rows are float whatever the dtype of q and of the pages
+    int out_float;
 };
 
 // how many keys back a query sees (0: all)
 __device__ __forceinline__ int seen_window(const AttnArgs& a) { return a.mask_window > 0 ? a.mask_window : a.window; }
+// the oldest key that a query at position qpos sees; it never decreases as qpos grows
+__device__ __forceinline__ int first_seen(const AttnArgs& a, int qpos) {
+    const int seen = seen_window(a);
+    int lo = seen > 0 ? max(0, qpos - seen + 1) : 0;
+    if (a.mask_chunk > 0) lo = max(lo, qpos / a.mask_chunk * a.mask_chunk);
+    return lo;
+}
 
 // ---- the order of a page's elements ---------------------------------------------------------
 // A page holds, per KV group, the keys K[64][d] and the values transposed V^T[d][64].  Pages of

@@ -36,7 +36,7 @@ __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
     float* alpha_s = Ps + AT_ROWS * PAGE_TOKENS;  // [AT_ROWS]
     float* l_s = alpha_s + AT_ROWS;             // [AT_ROWS]
     float* m_s = l_s + AT_ROWS;                 // [AT_ROWS]
-    __shared__ int row_tok[AT_ROWS], row_head[AT_ROWS], row_qpos[AT_ROWS];
+    __shared__ int row_tok[AT_ROWS], row_head[AT_ROWS], row_qpos[AT_ROWS], row_lo[AT_ROWS];
 
     const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
     const int R = a.H / a.G;
@@ -55,6 +55,7 @@ __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
             row_tok[tid] = seq;
             row_head[tid] = g * R + chunk * AT_ROWS + tid;
             row_qpos[tid] = work.qpos;
+            row_lo[tid] = first_seen(a, work.qpos);
         }
     } else {
         seq = a.tile_seq[blockIdx.x];
@@ -66,17 +67,17 @@ __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
             row_tok[tid] = a.cu_seqlens[seq] + q0 + tid;
             row_head[tid] = h;
             row_qpos[tid] = a.seq_pos0[seq] + q0 + tid;
+            row_lo[tid] = first_seen(a, a.seq_pos0[seq] + q0 + tid);
         }
     }
     __syncthreads();
     // visible key range of the tile: [lo, hi]
     const int qpos_first = row_qpos[0], qpos_last = row_qpos[n_rows - 1];
     const int hi = qpos_last;
-    const int seen = seen_window(a);
-    const int lo = seen > 0 ? max(0, qpos_first - seen + 1) : 0;
+    const int lo = row_lo[0];                                         // (the tile's first query sees furthest back)
     int page_lo = lo / PAGE_TOKENS, page_hi = hi / PAGE_TOKENS + 1;   // [page_lo, page_hi)
     if (a.decode) {
-        page_lo = work.page_lo;
+        page_lo = max(work.page_lo, page_lo);
         page_hi = work.page_hi;
     }
 
@@ -139,7 +140,7 @@ __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
             for (int i = 0; i < 4; ++i) {
                 const int r = 4 * wave + i;
                 const int qp = row_qpos[r];
-                const bool vis = r < n_rows && kpos <= qp && (seen <= 0 || qp - kpos < seen);
+                const bool vis = r < n_rows && kpos <= qp && kpos >= row_lo[r];
                 float sc = NEG_BIG;
                 if (vis) {
                     sc = s[i] * a.scale;
@@ -208,14 +209,15 @@ __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
             l = l * keep + expf(a.sink[head] - top);
         }
         const float inv = l > 0.f ? keep / l : 0.f;
-        T* o = (T*)a.out + (size_t)tok * a.H * dv + (size_t)head * dv;
+        const size_t at = (size_t)tok * a.H * dv + (size_t)head * dv;
         const float* gate = a.gate ? a.gate + (size_t)tok * a.gate_stride + (size_t)head * dv : nullptr;
 #pragma unroll
         for (int j = 0; j < MAXD / 16; ++j)
             if (j < n_cg) {
                 float y = acc[j] * inv;
                 if (gate) y *= 1.f / (1.f + expf(-gate[pc + 16 * j]));
-                o[pc + 16 * j] = from_f32<T>(y);
+                if (a.out_float) ((float*)a.out)[at + pc + 16 * j] = y;
+                else ((T*)a.out)[at + pc + 16 * j] = from_f32<T>(y);
             }
     }
 }
@@ -255,7 +257,11 @@ __global__ __launch_bounds__(MERGE_WAVES * WAVE) void attn_merge_kernel(AttnArgs
     float L = wave_sum(l);
     if (a.sink) L += expf(a.sink[head] - M);
     const float inv = L > 0.f ? 1.0f / L : 0.f;
-    T* o = (T*)a.out + (size_t)seq * H * d + (size_t)head * d;
+    const size_t at = (size_t)seq * H * d + (size_t)head * d;
+    auto store = [&](int c, float y) {
+        if (a.out_float) ((float*)a.out)[at + c] = y;
+        else ((T*)a.out)[at + c] = from_f32<T>(y);
+    };
     const float* gate = a.gate ? a.gate + (size_t)seq * a.gate_stride + (size_t)head * d : nullptr;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -267,13 +273,13 @@ __global__ __launch_bounds__(MERGE_WAVES * WAVE) void attn_merge_kernel(AttnArgs
             if (i < n_splits) acc += expf(p[(size_t)i * stride] - M) * early[i][j];
         for (int i = EARLY; i < n_splits; ++i) acc += expf(p[(size_t)i * stride] - M) * p[(size_t)i * stride + 2 + c];
         if (gate) acc *= 1.f / (1.f + expf(-gate[c]));
-        o[c] = from_f32<T>(acc * inv);
+        store(c, acc * inv);
     }
     for (int c = lane + 4 * WAVE; c < d; c += WAVE) {       // a head wider than 256
         float acc = 0.f;
         for (int i = 0; i < n_splits; ++i) acc += expf(p[(size_t)i * stride] - M) * p[(size_t)i * stride + 2 + c];
         if (gate) acc *= 1.f / (1.f + expf(-gate[c]));
-        o[c] = from_f32<T>(acc * inv);
+        store(c, acc * inv);
     }
 }
 
@@ -389,6 +395,8 @@ static void with_extras(AttnArgs& a, const picolm_attn_extras* x) {
     a.gate = x->gate;
     a.gate_stride = x->gate_stride;
     a.mask_window = x->mask_window;
+    a.mask_chunk = x->mask_chunk;
+    a.out_float = x->out_float;
 }
 
 static int check_extras(const char* who, const picolm_attn_extras* x, int H, int d) {
@@ -398,6 +406,7 @@ static int check_extras(const char* who, const picolm_attn_extras* x, int H, int
     const int dv = x->v_head_dim > 0 ? x->v_head_dim : d;
     PICOLM_REQUIRE(!x->gate || x->gate_stride >= H * dv, "%s: gate rows of %d floats for %d heads of %d", who, x->gate_stride, H, dv);
     PICOLM_REQUIRE(x->mask_window >= 0, "%s: a window of %d keys", who, x->mask_window);
+    PICOLM_REQUIRE(x->mask_chunk >= 0, "%s: stretches of %d keys", who, x->mask_chunk);
     return 0;
 }
 

@@ -85,7 +85,7 @@ __global__ __launch_bounds__(64 * PLAIN_WAVES) void attn_plain_mfma_kernel(AttnA
         tok = a.cu_seqlens[seq] + l, qpos = pos0 + l, qpos_first = pos0 + q0;
         slot = a.seq_slot[seq];
         hi = pos0 + min(q0 + 31, nnew - 1);
-        page_lo = decode_first_page(seen_window(a), qpos_first), page_hi = hi / PAGE_TOKENS + 1;      // (the tile's first query sees furthest back)
+        page_lo = first_seen(a, qpos_first) / PAGE_TOKENS, page_hi = hi / PAGE_TOKENS + 1;      // (the tile's first query sees furthest back)
     }
     // the wave's queries as operands: column `col`, k-step s covers elements 16 s + 8 h .. + 8
     bf16x8 Qf[D / 16];
@@ -113,9 +113,8 @@ __global__ __launch_bounds__(64 * PLAIN_WAVES) void attn_plain_mfma_kernel(AttnA
     const int tile_hi = min(2 * page_hi, hi / 32 + 1);       // tiles of 32 keys: this wave takes tile_lo, tile_lo + PLAIN_WAVES, ... below tile_hi
     const bool keys_in_turn = !a.waves_take_heads;           // the waves share one head's keys
     const int tile_step = keys_in_turn ? PLAIN_WAVES : 1;
-    // with a window, the tile of 32 keys that holds the oldest key any query of this wave sees
-    const int seen = seen_window(a);
-    const int oldest = seen > 0 ? max(0, qpos_first - seen + 1) : 0;
+    // with a window or stretches, the tile of 32 keys that holds the oldest key any query of this wave sees
+    const int oldest = first_seen(a, qpos_first), my_oldest = first_seen(a, qpos);
     const int tile_lo = max(2 * page_lo, oldest / 32) + (keys_in_turn ? wave : 0);
     // two sets of operands in turn: the loads of the tile after this one are queued before this
     // tile's products and stay there (the scheduler may not move them past the barrier), and the
@@ -152,7 +151,7 @@ __global__ __launch_bounds__(64 * PLAIN_WAVES) void attn_plain_mfma_kernel(AttnA
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
             const int key = key0 + key_of_elem(e, h);
-            const bool vis = q_ok && key <= qpos && (seen <= 0 || key > qpos - seen);
+            const bool vis = q_ok && key <= qpos && key >= my_oldest;
             S[e] = vis ? fmaf(S[e], scale2, bv[e]) : NEG_BIG;
             mx = fmaxf(mx, S[e]);
         }
@@ -246,7 +245,7 @@ __global__ __launch_bounds__(64 * PLAIN_WAVES) void attn_plain_mfma_kernel(AttnA
         l_run = l_run * keep + exp2_flushing(s2 - top);
     }
     const float inv = l_run > 0.f ? keep / l_run : 0.f;
-    bf16_t* o = (bf16_t*)a.out + (size_t)tok * a.H * DV + (size_t)head * DV;
+    const size_t at = (size_t)tok * a.H * DV + (size_t)head * DV;
     const float* gate = a.gate ? a.gate + (size_t)tok * a.gate_stride + (size_t)head * DV : nullptr;
 #pragma unroll
     for (int dt = 0; dt < DV / 32; ++dt)
@@ -255,7 +254,8 @@ __global__ __launch_bounds__(64 * PLAIN_WAVES) void attn_plain_mfma_kernel(AttnA
             const int c = 32 * dt + 8 * (e >> 2) + 4 * h + (e & 3);
             float y = O[dt][e] * inv;
             if (gate) y *= 1.f / (1.f + __expf(-gate[c]));
-            o[c] = from_f32<bf16_t>(y);
+            if (a.out_float) ((float*)a.out)[at + c] = y;
+            else ((bf16_t*)a.out)[at + c] = from_f32<bf16_t>(y);
         }
 }
 
@@ -292,6 +292,8 @@ static int fill_extras(const char* who, AttnArgs& a, const picolm_attn_extras* x
                    x->mask_window, a.window);
     a.bias = x->bias, a.bias_rows = x->bias_rows, a.sink = x->sink, a.gate = x->gate, a.gate_stride = x->gate_stride;
     a.mask_window = x->mask_window;
+    PICOLM_REQUIRE(x->mask_chunk >= 0, "%s: stretches of %d keys", who, x->mask_chunk);
+    a.mask_chunk = x->mask_chunk, a.out_float = x->out_float;
     return 0;
 }
 

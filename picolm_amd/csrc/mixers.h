@@ -25,26 +25,44 @@ typedef struct {
 } picolm_loop_input_args;
 int picolm_call_loop_input(void* user, const picolm_step_view* v);
 
-// Softmax attention over the cache entry with a norm of queries and keys, a bias by distance, a
-// sink and an output gate, each optional.
+// Softmax attention over the cache entry with biases of the projections, a rotation by position, a
+// norm of queries and keys, a bias by distance, a sink and an output gate, each optional.  A token's
+// q and k are prepared in this order: the projection's bias is added, the first rot_dims entries are
+// turned by the position, the norm is taken; values only get their bias.
 //   in: float rows [in_stride] holding q [H d], k [G d], v [G dv] and the gate's pre-activations
-//   [H dv] at the offsets named; out: rows [H dv] in the engine's dtype; extra[0]: scratch rows
+//   [H dv] at the offsets named (v_off may name the keys' place: the values are then the keys as
+//   projected); out: rows [H dv] in the engine's dtype (float with out_float); extra[0]: scratch rows
 //   [H d] in the engine's dtype.  Flags: PICOLM_CALL_KV | PICOLM_CALL_ATTENDS, partial_floats =
 //   H (dv + 2), tile_rows = picolm_attn_plain_mfma_tile_rows() where the engine runs in bfloat16 and
 //   picolm_attn_plain_mfma_takes(d, dv) (the matrix-core kernel then runs), else
 //   picolm_attn_prefill_tile_rows().  The operation writes its own pages: as plain arrays, or for the
 //   matrix-core kernel in the order of its operands.
+// maps > 1: a head's d entries are `maps` queries (and a KV head's `maps` keys) of d / maps entries
+//   side by side, each an attention of its own over the same values: query m of a head meets part m of
+//   the cached key.  The attention then runs over H maps heads: out rows [H maps][dv], scratch rows
+//   [H maps][d], partial_floats = H maps (dv + 2); norm and rotation cover each part by itself; no
+//   gate and no bias by distance; a sink has H maps entries.
 typedef struct {
     int32_t n_heads, n_kv_heads, head_dim, v_head_dim;
     int32_t in_stride, q_off, k_off, v_off, gate_off;     // gate_off < 0: no gate
     float scale, eps;
-    const float* q_norm;     // [head_dim] RMS norm of each query head (null: none), and of each key head
+    const float* q_norm;     // [head_dim / maps] RMS norm of each query head (null: none), and of each key head
     const float* k_norm;
     const float* bias;       // [H][bias_rows] by distance, the last entry for every distance beyond; null: none
     int32_t bias_rows;
     const float* sink;       // [H] or null
     int32_t window;          // > 0: a query sees its last `window` keys, no more than the cache entry's own window (which
                              // bounds the pages a step visits); 0: what the cache entry's window says
+    int32_t chunk;           // > 0: a query sees the keys of its own stretch of `chunk` positions (counted from the
+                             // sequence's first position) up to itself
+    int32_t maps;            // 0 or 1: one query a head
+    int32_t out_float;       // 1: the output rows are float
+    int32_t unit_qk;         // 1: queries and keys are divided by their root mean square (eps inside the root) where
+                             // q_norm / k_norm give no weight
+    const float* in_bias;    // [in_stride]: added to the input row where it is read (null: none)
+    const float* cos_table;  // [table_positions][rot_dims / 2]; null: no rotation
+    const float* sin_table;
+    int32_t table_positions, rot_dims, rot_half;      // rot_half = 1: entry i pairs with i + rot_dims / 2; 0: entry 2i with 2i + 1
 } picolm_sink_attention_args;
 int picolm_call_sink_attention(void* user, const picolm_step_view* v);
 
@@ -270,12 +288,32 @@ typedef struct {
 } picolm_rotate_heads_args;
 int picolm_call_rotate_heads(void* user, const picolm_step_view* v);
 
+// out[c] += in[c] + vec[c] over `width` columns of float rows: what a pass over a looped stretch of
+// layers adds before its first layer (the embedding's rows again, and the pass's vector), or any
+// other sum of rows.  in: float rows [width] or absent; vec: [width] or null.
+typedef struct {
+    const float* vec;
+    int32_t width;
+} picolm_add_rows_args;
+int picolm_call_add_rows(void* user, const picolm_step_view* v);
+
+// Two attention maps a head become one: o = a1 - lambda a2, divided by its root mean square over the
+// head's `vdim` values (eps inside the root, no weight), times `mult`.
+//   in: float rows [heads][2][vdim], map m of head h at (2 h + m) vdim; out: rows [heads vdim] of out_dtype.
+typedef struct {
+    int32_t heads, vdim, out_dtype;
+    float lambda, eps, mult;
+} picolm_map_difference_args;
+int picolm_call_map_difference(void* user, const picolm_step_view* v);
+
 // ---- a routed feed-forward ---------------------------------------------------------------------
 // Each row picks `top` of its `experts` router outputs (ties: the lower index).
 //   scoring 0: the largest logits + bias are picked, weighted by the softmax over the picked
 //              (biased) logits alone;
 //   scoring 1: s = softmax over all the logits; the largest s + bias are picked; the weights are
 //              the picked s over their sum (+ 1e-20), times `scale`.
+//   scoring 2: s = sigmoid(logit); the largest s + bias are picked; the weights are the picked s
+//              themselves, times `scale`.
 //   in: float rows [in_stride] (0: experts) whose first `experts` entries are the router logits
 //   without bias; out: rows of 2 top words: the picked outputs (int32) and then their weights (float).
 typedef struct {
@@ -302,6 +340,10 @@ typedef struct {
     int32_t experts, top, width, ff;
     int32_t adds;            // 1: out += the sum; 0: out = the sum
     int32_t identity;        // picks from `experts` up to experts + identity give the row itself
+    int32_t act;             // 0: silu(g) * u.  1: g' = min(g, limit), u' = clamp(u, -limit, limit), g' sigmoid(alpha g') (u' + 1)
+    float limit, alpha;
+    int32_t weight_on_input; // 1: a pick's weight multiplies what its expert reads (g and u before the activation), and the
+                             // sum over a row's picks is plain
 } picolm_routed_experts_args;
 int picolm_call_routed_experts(void* user, const picolm_step_view* v);
 

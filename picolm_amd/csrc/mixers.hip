@@ -49,43 +49,94 @@ extern "C" int picolm_call_loop_input(void* user, const picolm_step_view* v) {
 }
 
 // ---- attention with a norm of queries and keys, a bias by distance, a sink and a gate ------------
-// One wave per (token, head): query heads go, normed, to the rows the attention kernel reads;
-// key heads, normed, and value heads to the token's place in its cache page (K[G][64][d],
-// V^T[G][dv][64] as plain arrays, or with `tiled` in the order of the MFMA operands).
+struct QkPrepare {
+    const float* in;
+    int in_stride, q_off, k_off, v_off;
+    const float* q_norm;
+    const float* k_norm;
+    float eps;
+    int unit_qk;
+    const float* in_bias;
+    const float* cos_t;
+    const float* sin_t;
+    int table_positions, rot_dims, rot_half;
+    const int32_t* tok_pos;
+    const int32_t* write_pages;
+    int H, G, d, dv, maps;
+    bool tiled;
+};
+
+// One wave per (token, part): a part is one of the `maps` queries of a query head, one of the `maps`
+// keys of a KV head, or a value head.  Queries go, biased, turned and normed, to the rows the
+// attention kernel reads (query m of a head as a row of d entries that is zero outside part m, so
+// that its product with the cached key is its product with the key's part m); keys likewise to the
+// token's place in its cache page, values (biased only) too (K[G][64][d], V^T[G][dv][64] as plain
+// arrays, or with `tiled` in the order of the MFMA operands).
 template <typename T>
-__global__ void qk_norm_store_kernel(const float* __restrict__ in, int in_stride, int q_off, int k_off, int v_off, T* __restrict__ q_out,
-                                     T* __restrict__ k_pages, T* __restrict__ v_pages, const float* __restrict__ q_norm,
-                                     const float* __restrict__ k_norm, float eps, const int32_t* __restrict__ tok_pos,
-                                     const int32_t* __restrict__ write_pages, int H, int G, int d, int dv, bool tiled) {
+__global__ void qk_norm_store_kernel(QkPrepare a, T* __restrict__ q_out, T* __restrict__ k_pages, T* __restrict__ v_pages) {
     const size_t row = blockIdx.x;
     const int unit = blockIdx.y, lane = threadIdx.x;
-    const float* src = in + row * in_stride;
-    if (unit < H + G) {
-        const bool is_q = unit < H;
-        const int head = is_q ? unit : unit - H;
-        const float* x = src + (is_q ? q_off : k_off) + (size_t)head * d;
-        const float* w = is_q ? q_norm : k_norm;
+    const int H = a.H, G = a.G, d = a.d, dv = a.dv, maps = a.maps, dp = d / maps;
+    const float* src = a.in + row * a.in_stride;
+    if (unit < (H + G) * maps) {
+        const bool is_q = unit < H * maps;
+        const int part = is_q ? unit : unit - H * maps;          // (head, map) counted together
+        const int at = (is_q ? a.q_off : a.k_off) + part * dp;
+        const float* x = src + at;
+        const float* b = a.in_bias ? a.in_bias + at : nullptr;
+        const float* w = is_q ? a.q_norm : a.k_norm;
+        const int half = a.rot_dims / 2;
+        const int pos = a.cos_t ? min(a.tok_pos[row], a.table_positions - 1) : 0;
+        const float* ct = a.cos_t ? a.cos_t + (size_t)pos * half : nullptr;
+        const float* st = a.cos_t ? a.sin_t + (size_t)pos * half : nullptr;
+        auto entry = [&](int i) { return b ? x[i] + b[i] : x[i]; };
+        auto value = [&](int i) {
+            if (!ct || i >= a.rot_dims) return entry(i);
+            int j, first, second;
+            if (a.rot_half) j = i < half ? i : i - half, first = j, second = j + half;
+            else j = i >> 1, first = 2 * j, second = 2 * j + 1;
+            const float u = entry(first), v = entry(second), c = ct[j], s = st[j];
+            return i == first ? u * c - v * s : v * c + u * s;
+        };
         float inv = 1.f;
-        if (w) {
+        const bool norms = w || a.unit_qk;
+        if (norms) {
             float ssq = 0.f;
-            for (int i = lane; i < d; i += WAVE) ssq += x[i] * x[i];
+            for (int i = lane; i < dp; i += WAVE) {
+                const float y = value(i);
+                ssq += y * y;
+            }
             ssq = wave_sum(ssq);
-            inv = 1.f / sqrtf(ssq / (float)d + eps);
+            inv = 1.f / sqrtf(ssq / (float)dp + a.eps);
         }
+        const int m = part % maps, lo = m * dp;
         if (is_q) {
-            T* dst = q_out + (row * H + head) * d;
-            for (int i = lane; i < d; i += WAVE) dst[i] = from_f32<T>(w ? x[i] * inv * w[i] : x[i]);
+            T* dst = q_out + (row * H * maps + part) * d;
+            for (int i = lane; i < d; i += WAVE) {
+                float y = 0.f;
+                if (i >= lo && i < lo + dp) {
+                    y = value(i - lo);
+                    if (norms) y = w ? y * inv * w[i - lo] : y * inv;
+                }
+                dst[i] = from_f32<T>(y);
+            }
         } else {
-            const int key = tok_pos[row] % PAGE_TOKENS;
-            T* dst = k_pages + ((size_t)write_pages[row] * G + head) * PAGE_TOKENS * d;
-            for (int i = lane; i < d; i += WAVE) dst[k_page_offset(key, i, d, tiled)] = from_f32<T>(w ? x[i] * inv * w[i] : x[i]);
+            const int head = part / maps;
+            const int key = a.tok_pos[row] % PAGE_TOKENS;
+            T* dst = k_pages + ((size_t)a.write_pages[row] * G + head) * PAGE_TOKENS * d;
+            for (int i = lane; i < dp; i += WAVE) {
+                float y = value(i);
+                if (norms) y = w ? y * inv * w[i] : y * inv;
+                dst[k_page_offset(key, lo + i, d, a.tiled)] = from_f32<T>(y);
+            }
         }
     } else {
-        const int head = unit - H - G;
-        const float* x = src + v_off + (size_t)head * dv;
-        const int key = tok_pos[row] % PAGE_TOKENS;
-        T* dst = v_pages + ((size_t)write_pages[row] * G + head) * dv * PAGE_TOKENS;
-        for (int i = lane; i < dv; i += WAVE) dst[v_page_offset(i, key, dv, tiled)] = from_f32<T>(x[i]);
+        const int head = unit - (H + G) * maps;
+        const float* x = src + a.v_off + (size_t)head * dv;
+        const float* b = a.in_bias ? a.in_bias + a.v_off + (size_t)head * dv : nullptr;
+        const int key = a.tok_pos[row] % PAGE_TOKENS;
+        T* dst = v_pages + ((size_t)a.write_pages[row] * G + head) * dv * PAGE_TOKENS;
+        for (int i = lane; i < dv; i += WAVE) dst[v_page_offset(i, key, dv, a.tiled)] = from_f32<T>(b ? x[i] + b[i] : x[i]);
     }
 }
 
@@ -95,6 +146,7 @@ extern "C" int picolm_call_sink_attention(void* user, const picolm_step_view* v)
     PICOLM_REQUIRE(a && v->in && v->out && v->extra[0] && v->k_pages && v->v_pages && v->page_table,
                    "sink_attention: buffers or the cache entry are missing");
     const int H = a->n_heads, G = a->n_kv_heads, d = a->head_dim, dv = a->v_head_dim, dt = v->dtype, es = elem_bytes(dt);
+    const int maps = a->maps > 1 ? a->maps : 1;
     PICOLM_REQUIRE(H > 0 && G > 0 && H % G == 0 && d > 0 && dv > 0, "sink_attention: %d heads over %d, sizes %d and %d", H, G, d, dv);
     PICOLM_REQUIRE(G == v->n_kv_heads && d == v->head_dim && dv == v->v_head_dim && v->window >= 0,
                    "sink_attention: the cache entry holds %d heads of %d and %d (window %d), the operation has %d of %d and %d", v->n_kv_heads,
@@ -103,23 +155,28 @@ extern "C" int picolm_call_sink_attention(void* user, const picolm_step_view* v)
                        a->k_off + G * d <= a->in_stride && a->v_off >= 0 && a->v_off + G * dv <= a->in_stride &&
                        (a->gate_off < 0 || a->gate_off + H * dv <= a->in_stride),
                    "sink_attention: the input rows of %d floats do not hold what the offsets name", a->in_stride);
-    PICOLM_REQUIRE(v->out_row_bytes >= H * dv * es && v->extra_row_bytes[0] >= H * d * es, "sink_attention: output or scratch rows too short");
+    PICOLM_REQUIRE(d % maps == 0 && (maps == 1 || (a->gate_off < 0 && !a->bias)),
+                   "sink_attention: %d queries a head of %d entries (with several there is no gate and no bias by distance)", maps, d);
+    PICOLM_REQUIRE(v->out_row_bytes >= (int64_t)H * maps * dv * (a->out_float ? 4 : es) && v->extra_row_bytes[0] >= (int64_t)H * maps * d * es,
+                   "sink_attention: output or scratch rows too short");
     PICOLM_REQUIRE(!v->kv_writes || v->write_pages, "sink_attention: no pages to write to");
     PICOLM_REQUIRE(a->window >= 0 && (v->window <= 0 || a->window <= v->window), "sink_attention: a window of %d keys over a cache entry laid out for %d",
                    a->window, v->window);
-    PICOLM_REQUIRE(H + G + G <= 65535, "sink_attention: %d heads exceed the grid", H + 2 * G);
+    PICOLM_REQUIRE(a->chunk >= 0, "sink_attention: stretches of %d keys", a->chunk);
+    PICOLM_REQUIRE(!a->cos_table || (a->sin_table && a->table_positions > 0 && a->rot_dims > 0 && a->rot_dims % 2 == 0 && a->rot_dims <= d / maps),
+                   "sink_attention: a rotation of %d entries of %d, tables for %d positions", a->rot_dims, d / maps, a->table_positions);
+    PICOLM_REQUIRE((H + G) * maps + G <= 65535, "sink_attention: %d heads exceed the grid", (H + G) * maps + G);
     if (v->n_tokens <= 0) return 0;
     const float* in = (const float*)v->in;
-    dim3 grid(v->n_tokens, v->kv_writes ? H + 2 * G : H);
+    dim3 grid(v->n_tokens, v->kv_writes ? (H + G) * maps + G : H * maps);
     const bool mfma = dt == PICOLM_BF16 && picolm_attn_plain_mfma_takes(d, dv);      // then the pages are in the matrix-core kernel's order
+    QkPrepare p = {in, a->in_stride, a->q_off, a->k_off, a->v_off, a->q_norm, a->k_norm, a->eps, a->unit_qk, a->in_bias, a->cos_table,
+                   a->sin_table, a->table_positions, a->rot_dims, a->rot_half, v->tok_pos, v->write_pages, H, G, d, dv, maps,
+                   dt == PICOLM_BF16 && mfma};
     if (dt == PICOLM_F32)
-        qk_norm_store_kernel<float><<<grid, WAVE, 0, v->stream>>>(in, a->in_stride, a->q_off, a->k_off, a->v_off, (float*)v->extra[0],
-                                                                  (float*)v->k_pages, (float*)v->v_pages, a->q_norm, a->k_norm, a->eps,
-                                                                  v->tok_pos, v->write_pages, H, G, d, dv, false);
+        qk_norm_store_kernel<float><<<grid, WAVE, 0, v->stream>>>(p, (float*)v->extra[0], (float*)v->k_pages, (float*)v->v_pages);
     else
-        qk_norm_store_kernel<bf16_t><<<grid, WAVE, 0, v->stream>>>(in, a->in_stride, a->q_off, a->k_off, a->v_off, (bf16_t*)v->extra[0],
-                                                                   (bf16_t*)v->k_pages, (bf16_t*)v->v_pages, a->q_norm, a->k_norm, a->eps,
-                                                                   v->tok_pos, v->write_pages, H, G, d, dv, mfma);
+        qk_norm_store_kernel<bf16_t><<<grid, WAVE, 0, v->stream>>>(p, (bf16_t*)v->extra[0], (bf16_t*)v->k_pages, (bf16_t*)v->v_pages);
     PICOLM_LAUNCH_CHECK("sink_attention (norm and cache write)");
     picolm_attn_extras x;
     x.v_head_dim = dv;
@@ -129,25 +186,28 @@ extern "C" int picolm_call_sink_attention(void* user, const picolm_step_view* v)
     x.gate = a->gate_off >= 0 ? in + a->gate_off : nullptr;
     x.gate_stride = a->in_stride;
     x.mask_window = a->window;
+    x.mask_chunk = a->chunk;
+    x.out_float = a->out_float;
+    const int HM = H * maps;
     if (mfma && v->is_decode)
         return picolm_attn_decode_plain_mfma(v->extra[0], v->k_pages, v->v_pages, v->out, v->partial, v->n_seq, v->chunk_list, v->n_chunks,
-                                             v->pages_per_chunk, v->most_chunks, v->seq_pos0, v->page_table, v->max_pages, v->ring_pages, H,
+                                             v->pages_per_chunk, v->most_chunks, v->seq_pos0, v->page_table, v->max_pages, v->ring_pages, HM,
                                              G, d, v->window, a->scale, &x, v->stream);
     if (mfma) {
         PICOLM_REQUIRE(v->tile_seq && v->tile_rows == picolm_attn_plain_mfma_tile_rows(), "sink_attention: the step has no tiles of %d rows",
                        picolm_attn_plain_mfma_tile_rows());
         return picolm_attn_prefill_plain_mfma(v->extra[0], v->k_pages, v->v_pages, v->out, v->tile_seq, v->tile_q0, v->n_tiles, v->seq_slot,
-                                              v->seq_pos0, v->seq_nnew, v->cu_seqlens, v->page_table, v->max_pages, v->ring_pages, H, G, d,
+                                              v->seq_pos0, v->seq_nnew, v->cu_seqlens, v->page_table, v->max_pages, v->ring_pages, HM, G, d,
                                               v->window, a->scale, &x, v->stream);
     }
     if (v->is_decode)
         return picolm_attn_decode_plain(v->extra[0], v->k_pages, v->v_pages, v->out, v->partial, dt, v->n_seq, v->chunk_list, v->n_chunks,
-                                        v->pages_per_chunk, v->most_chunks, v->seq_pos0, v->page_table, v->max_pages, v->ring_pages, H, G, d,
+                                        v->pages_per_chunk, v->most_chunks, v->seq_pos0, v->page_table, v->max_pages, v->ring_pages, HM, G, d,
                                         v->window, a->scale, &x, v->stream);
     PICOLM_REQUIRE(v->tile_seq && v->tile_rows == picolm_attn_prefill_tile_rows(), "sink_attention: the step has no tiles of %d rows",
                    picolm_attn_prefill_tile_rows());
     return picolm_attn_prefill_plain(v->extra[0], v->k_pages, v->v_pages, v->out, dt, v->tile_seq, v->tile_q0, v->n_tiles, v->seq_slot,
-                                     v->seq_pos0, v->seq_nnew, v->cu_seqlens, v->page_table, v->max_pages, v->ring_pages, H, G, d, v->window,
+                                     v->seq_pos0, v->seq_nnew, v->cu_seqlens, v->page_table, v->max_pages, v->ring_pages, HM, G, d, v->window,
                                      a->scale, &x, v->stream);
 }
 

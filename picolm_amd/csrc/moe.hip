@@ -30,6 +30,25 @@ __global__ void route_top_kernel(const float* __restrict__ logits, int in_stride
     const float* z = logits + (size_t)row * in_stride;
     int32_t* ids = out + (size_t)row * 2 * top;
     float* w = (float*)(ids + top);
+    if (scoring == 2) {
+        // s = sigmoid of every output; the picks are the largest s + bias, their weights the picked s themselves
+        float last_c = INFINITY;
+        int last_e = -1;
+        for (int k = 0; k < top; ++k) {
+            float best = -INFINITY, best_s = 0.f;
+            int be = -1;
+            for (int e = 0; e < E; ++e) {
+                const float se = 1.f / (1.f + expf(-z[e])), ce = se + (bias ? bias[e] : 0.f);
+                const bool after_last = ce < last_c || (ce == last_c && e > last_e);
+                if (after_last && (be < 0 || ce > best)) best = ce, be = e, best_s = se;
+            }
+            if (be < 0) be = k % E, best = -INFINITY, best_s = 0.f;     // (only logits that are no numbers lead here)
+            ids[k] = be;
+            w[k] = best_s * scale;
+            last_c = best, last_e = be;
+        }
+        return;
+    }
     if (scoring == 1) {
         // s = softmax over every output; the picks are the largest s + bias, their weights the picked s over their sum
         float zmax = -INFINITY, den = 0.f;
@@ -82,7 +101,7 @@ extern "C" int picolm_call_route_top(void* user, const picolm_step_view* v) {
                    a ? a->top : 0, a ? a->experts : 0);
     const int in_stride = a->in_stride ? a->in_stride : a->experts;
     PICOLM_REQUIRE(in_stride >= a->experts && v->in_row_bytes >= (int64_t)in_stride * 4 && v->out_row_bytes >= 2 * a->top * 4, "route_top: rows too short");
-    PICOLM_REQUIRE(a->scoring == 0 || a->scoring == 1, "route_top: scoring %d is not known", a->scoring);
+    PICOLM_REQUIRE(a->scoring >= 0 && a->scoring <= 2, "route_top: scoring %d is not known", a->scoring);
     if (v->rows <= 0) return 0;
     route_top_kernel<<<ceil_div(v->rows, 64), 64, 0, v->stream>>>((const float*)v->in, in_stride, a->bias, (int32_t*)v->out, a->experts, a->top,
                                                                  v->rows, a->scoring, a->scale);
@@ -125,16 +144,33 @@ template <> __device__ __forceinline__ float lane_dot<float>(const float* __rest
 
 #define MOE_UNITS 16     // hidden units, or outputs, a workgroup of four waves takes
 
+// what an expert's hidden unit is, from its two products g and u (mixers.h: picolm_routed_experts_args.act)
+struct ExpertAct {
+    int kind;
+    float limit, alpha;
+    int weight_on_input;
+};
+__device__ __forceinline__ float expert_act(const ExpertAct& x, float g, float u) {
+    if (x.kind == 1) {
+        g = fminf(g, x.limit);
+        u = fminf(fmaxf(u, -x.limit), x.limit);
+        return g / (1.f + expf(-x.alpha * g)) * (u + 1.f);
+    }
+    return g / (1.f + expf(-g)) * u;
+}
+
 // act[row][pick][f] = silu(W_gate[e][f] . h) * (W_up[e][f] . h); a wave has its four units' eight rows on their way at once
 template <typename TW, typename TH>
 __global__ __launch_bounds__(256) void expert_hidden_kernel(const TH* __restrict__ h, const int32_t* __restrict__ picks, float* __restrict__ act,
-                                                            const TW* __restrict__ gate, const TW* __restrict__ up, int E, int top, int D, int F) {
+                                                            const TW* __restrict__ gate, const TW* __restrict__ up, int E, int top, int D, int F,
+                                                            ExpertAct xa) {
     extern __shared__ float moe_lds[];       // [D]
     const int pair = blockIdx.x, row = pair / top, k = pair % top;
     const int e = picks[(size_t)row * 2 * top + k];
     for (int c = threadIdx.x; c < D; c += blockDim.x) moe_lds[c] = to_f32<TH>(h[(size_t)row * D + c]);
     __syncthreads();
     if (e < 0 || e >= E) return;
+    const float on_input = xa.weight_on_input ? ((const float*)(picks + (size_t)row * 2 * top + top))[k] : 1.f;
     const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
     const int f0 = blockIdx.y * MOE_UNITS + wave * 4;
     float g[4], u[4];
@@ -146,8 +182,8 @@ __global__ __launch_bounds__(256) void expert_hidden_kernel(const TH* __restrict
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        const float gs = wave_sum(g[j]), us = wave_sum(u[j]);
-        if (lane == 0 && f0 + j < F) act[((size_t)row * top + k) * F + f0 + j] = gs / (1.f + expf(-gs)) * us;
+        const float gs = wave_sum(g[j]) * on_input, us = wave_sum(u[j]) * on_input;
+        if (lane == 0 && f0 + j < F) act[((size_t)row * top + k) * F + f0 + j] = expert_act(xa, gs, us);
     }
 }
 
@@ -163,7 +199,7 @@ __device__ __forceinline__ float identity_weight(const int32_t* ids, const float
 template <typename TW, typename TH>
 __global__ __launch_bounds__(256) void expert_down_kernel(const float* __restrict__ act, const int32_t* __restrict__ picks, float* __restrict__ out,
                                                           const TW* __restrict__ down, int E, int top, int D, int F, int adds,
-                                                          const TH* __restrict__ h, int identity) {
+                                                          const TH* __restrict__ h, int identity, int plain_sum) {
     extern __shared__ float moe_lds[];       // [top][F]
     const int row = blockIdx.x;
     for (int c = threadIdx.x; c < top * F; c += blockDim.x) moe_lds[c] = act[(size_t)row * top * F + c];
@@ -180,7 +216,7 @@ __global__ __launch_bounds__(256) void expert_down_kernel(const float* __restric
 #pragma unroll
         for (int j = 0; j < 4; ++j) part[j] = lane_dot<TW>(down + ((size_t)e * D + min(d0 + j, D - 1)) * F, moe_lds + (size_t)k * F, F, lane);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) total[j] += w[k] * wave_sum(part[j]);
+        for (int j = 0; j < 4; ++j) total[j] += (plain_sum ? 1.f : w[k]) * wave_sum(part[j]);
     }
     const float same = identity > 0 ? identity_weight(ids, w, top, E, identity) : 0.f;
 #pragma unroll
@@ -254,7 +290,7 @@ __device__ __forceinline__ int tile_of(const int32_t* __restrict__ plan, int E, 
 template <bool HIDDEN>
 __global__ __launch_bounds__(256) void grouped_tile_kernel(const bf16_t* __restrict__ a, const int32_t* __restrict__ plan, void* __restrict__ out,
                                                            const bf16_t* __restrict__ w0, const bf16_t* __restrict__ w1, int E, int top, int K,
-                                                           int N) {
+                                                           int N, const int32_t* __restrict__ picks, ExpertAct xa) {
     constexpr int NB = HIDDEN ? 2 : 1;
     __shared__ int32_t pairs[GM_ROWS];
     __shared__ __attribute__((aligned(16))) bf16_t As[GM_ROWS * GM_LD];
@@ -321,8 +357,8 @@ __global__ __launch_bounds__(256) void grouped_tile_kernel(const bf16_t* __restr
             const int pair = pairs[rh * 64 + i * 32 + 8 * (q / 4) + q % 4 + 4 * kq];
             if (pair < 0) continue;
             if constexpr (HIDDEN) {
-                const float g = acc[i][0][q];
-                ((bf16_t*)out)[(size_t)pair * N + n] = f32_to_bf16_bits(g / (1.f + expf(-g)) * acc[i][NB - 1][q]);
+                const float on_input = xa.weight_on_input ? ((const float*)(picks + (size_t)(pair / top) * 2 * top + top))[pair % top] : 1.f;
+                ((bf16_t*)out)[(size_t)pair * N + n] = f32_to_bf16_bits(expert_act(xa, acc[i][0][q] * on_input, acc[i][NB - 1][q] * on_input));
             } else {
                 ((float*)out)[(size_t)pair * N + n] = acc[i][0][q];
             }
@@ -331,7 +367,7 @@ __global__ __launch_bounds__(256) void grouped_tile_kernel(const bf16_t* __restr
 
 // out[row] (+)= sum_k w[row][k] y[row][k], in the order of the picks
 __global__ void grouped_sum_kernel(const float* __restrict__ y, const int32_t* __restrict__ picks, float* __restrict__ out, int E, int top, int D,
-                                   int adds, const bf16_t* __restrict__ h, int identity) {
+                                   int adds, const bf16_t* __restrict__ h, int identity, int plain_sum) {
     const size_t row = blockIdx.x;
     const int32_t* ids = picks + row * 2 * top;
     const float* w = (const float*)(ids + top);
@@ -339,7 +375,7 @@ __global__ void grouped_sum_kernel(const float* __restrict__ y, const int32_t* _
     for (int d = threadIdx.x; d < D; d += blockDim.x) {
         float total = 0.f;
         for (int k = 0; k < top; ++k)
-            if (ids[k] >= 0 && ids[k] < E) total += w[k] * y[(row * top + k) * D + d];
+            if (ids[k] >= 0 && ids[k] < E) total += (plain_sum ? 1.f : w[k]) * y[(row * top + k) * D + d];
         out[row * D + d] = (adds ? out[row * D + d] : 0.f) + total + (same != 0.f ? same * bf16_bits_to_f32(h[row * D + d]) : 0.f);
     }
 }
@@ -357,6 +393,10 @@ extern "C" int picolm_call_routed_experts(void* user, const picolm_step_view* v)
     PICOLM_REQUIRE(v->in_row_bytes >= D * elem_bytes(v->dtype) && v->out_row_bytes >= D * 4 && v->extra_row_bytes[0] >= 2 * top * 4 &&
                        v->extra_row_bytes[1] >= (int64_t)top * F * 4,
                    "routed_experts: rows too short for a width of %d, %d picks and %d hidden units", D, top, F);
+    PICOLM_REQUIRE(a->act == 0 || (a->act == 1 && a->limit > 0.f), "routed_experts: activation %d (limit %g) is not known", a->act, (double)a->limit);
+    PICOLM_REQUIRE(!a->weight_on_input || a->identity == 0, "routed_experts: weights on the experts' input and picks that give the input back do not go together");
+    const ExpertAct xa = {a->act, a->limit, a->alpha, a->weight_on_input};
+    const int plain_sum = a->weight_on_input ? 1 : 0;
     const size_t lds_a = sizeof(float) * (size_t)D, lds_b = sizeof(float) * (size_t)top * F;
     PICOLM_REQUIRE(lds_a <= 64 * 1024 && lds_b <= 64 * 1024, "routed_experts: a width of %d or %d picks of %d hidden units exceed 64 KiB of LDS", D,
                    top, F);
@@ -376,34 +416,34 @@ extern "C" int picolm_call_routed_experts(void* user, const picolm_step_view* v)
         PICOLM_LAUNCH_CHECK("routed_experts (plan)");
         const unsigned tiles = (unsigned)(ceil_div64(n_pairs, GM_ROWS) + E);      // no more than these are filled; the rest leave at once
         grouped_tile_kernel<true><<<dim3(tiles, ceil_div(F, GM_COLS)), 256, 0, v->stream>>>((const bf16_t*)v->in, plan, act, (const bf16_t*)a->gate,
-                                                                                           (const bf16_t*)a->up, E, top, D, F);
+                                                                                           (const bf16_t*)a->up, E, top, D, F, picks, xa);
         PICOLM_LAUNCH_CHECK("routed_experts (hidden, grouped)");
         grouped_tile_kernel<false><<<dim3(tiles, ceil_div(D, GM_COLS)), 256, 0, v->stream>>>((const bf16_t*)act, plan, y, (const bf16_t*)a->down,
-                                                                                            nullptr, E, top, F, D);
+                                                                                            nullptr, E, top, F, D, picks, xa);
         PICOLM_LAUNCH_CHECK("routed_experts (down, grouped)");
-        grouped_sum_kernel<<<v->rows, 256, 0, v->stream>>>(y, picks, (float*)v->out, E, top, D, a->adds, (const bf16_t*)v->in, a->identity);
+        grouped_sum_kernel<<<v->rows, 256, 0, v->stream>>>(y, picks, (float*)v->out, E, top, D, a->adds, (const bf16_t*)v->in, a->identity, plain_sum);
         PICOLM_LAUNCH_CHECK("routed_experts (sum)");
         return 0;
     }
     const dim3 grid_a((unsigned)(v->rows * top), ceil_div(F, MOE_UNITS)), grid_b(v->rows, ceil_div(D, MOE_UNITS));
     if (a->weight_dt == PICOLM_F32 && v->dtype == PICOLM_F32) {
         expert_hidden_kernel<float, float><<<grid_a, 256, lds_a, v->stream>>>((const float*)v->in, picks, act, (const float*)a->gate,
-                                                                              (const float*)a->up, E, top, D, F);
+                                                                              (const float*)a->up, E, top, D, F, xa);
         PICOLM_LAUNCH_CHECK("routed_experts (hidden)");
         expert_down_kernel<float, float><<<grid_b, 256, lds_b, v->stream>>>(act, picks, (float*)v->out, (const float*)a->down, E, top, D, F, a->adds,
-                                                                            (const float*)v->in, a->identity);
+                                                                            (const float*)v->in, a->identity, plain_sum);
     } else if (a->weight_dt == PICOLM_F32) {
         expert_hidden_kernel<float, bf16_t><<<grid_a, 256, lds_a, v->stream>>>((const bf16_t*)v->in, picks, act, (const float*)a->gate,
-                                                                               (const float*)a->up, E, top, D, F);
+                                                                               (const float*)a->up, E, top, D, F, xa);
         PICOLM_LAUNCH_CHECK("routed_experts (hidden)");
         expert_down_kernel<float, bf16_t><<<grid_b, 256, lds_b, v->stream>>>(act, picks, (float*)v->out, (const float*)a->down, E, top, D, F, a->adds,
-                                                                             (const bf16_t*)v->in, a->identity);
+                                                                             (const bf16_t*)v->in, a->identity, plain_sum);
     } else {
         expert_hidden_kernel<bf16_t, bf16_t><<<grid_a, 256, lds_a, v->stream>>>((const bf16_t*)v->in, picks, act, (const bf16_t*)a->gate,
-                                                                                (const bf16_t*)a->up, E, top, D, F);
+                                                                                (const bf16_t*)a->up, E, top, D, F, xa);
         PICOLM_LAUNCH_CHECK("routed_experts (hidden)");
         expert_down_kernel<bf16_t, bf16_t><<<grid_b, 256, lds_b, v->stream>>>(act, picks, (float*)v->out, (const bf16_t*)a->down, E, top, D, F, a->adds,
-                                                                              (const bf16_t*)v->in, a->identity);
+                                                                              (const bf16_t*)v->in, a->identity, plain_sum);
     }
     PICOLM_LAUNCH_CHECK("routed_experts (down)");
     return 0;

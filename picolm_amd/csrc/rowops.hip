@@ -537,3 +537,61 @@ extern "C" int picolm_call_rotate_heads(void* user, const picolm_step_view* v) {
     PICOLM_LAUNCH_CHECK("rotate_heads");
     return 0;
 }
+
+// ---- a sum of rows -----------------------------------------------------------------------------------
+__global__ void add_rows_kernel(float* __restrict__ x, const float* __restrict__ in, const float* __restrict__ vec, int W) {
+    const size_t row = blockIdx.x;
+    for (int c = threadIdx.x; c < W; c += blockDim.x) {
+        float y = x[row * W + c];
+        if (in) y += in[row * W + c];
+        if (vec) y += vec[c];
+        x[row * W + c] = y;
+    }
+}
+
+extern "C" int picolm_call_add_rows(void* user, const picolm_step_view* v) {
+    const picolm_add_rows_args* a = (const picolm_add_rows_args*)user;
+    VIEW_REQUIRE("add_rows", v);
+    PICOLM_REQUIRE(a && a->width > 0 && v->out && (v->in || a->vec), "add_rows: nothing to add, or no rows to add to");
+    PICOLM_REQUIRE(v->out_row_bytes >= a->width * 4 && (!v->in || v->in_row_bytes >= a->width * 4), "add_rows: rows too short for a width of %d",
+                   a->width);
+    if (v->rows <= 0) return 0;
+    add_rows_kernel<<<v->rows, 256, 0, v->stream>>>((float*)v->out, (const float*)v->in, a->vec, a->width);
+    PICOLM_LAUNCH_CHECK("add_rows");
+    return 0;
+}
+
+// ---- two attention maps a head become one ------------------------------------------------------------
+// one wave per (row, head)
+__global__ void map_difference_kernel(const float* __restrict__ in, void* __restrict__ out, int out_dt, int heads, int dv, float lambda, float eps,
+                                      float mult) {
+    const size_t row = blockIdx.x;
+    const int head = blockIdx.y * (blockDim.x / WAVE) + threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    if (head >= heads) return;
+    const float* a1 = in + (row * heads + head) * 2 * dv;
+    const float* a2 = a1 + dv;
+    float ssq = 0.f;
+    for (int c = lane; c < dv; c += WAVE) {
+        const float o = a1[c] - lambda * a2[c];
+        ssq += o * o;
+    }
+    ssq = wave_sum(ssq);
+    const float k = mult / sqrtf(ssq / (float)dv + eps);
+    for (int c = lane; c < dv; c += WAVE) store_from_f32(out, (row * heads + head) * dv + c, out_dt, (a1[c] - lambda * a2[c]) * k);
+}
+
+extern "C" int picolm_call_map_difference(void* user, const picolm_step_view* v) {
+    const picolm_map_difference_args* a = (const picolm_map_difference_args*)user;
+    VIEW_REQUIRE("map_difference", v);
+    PICOLM_REQUIRE(a && a->heads > 0 && a->vdim > 0 && known_dtype(a->out_dtype) && v->in && v->out && v->in != v->out,
+                   "map_difference: sizes or buffers are missing (input and output differ)");
+    PICOLM_REQUIRE(v->in_row_bytes >= (int64_t)a->heads * 2 * a->vdim * 4 && v->out_row_bytes >= (int64_t)a->heads * a->vdim * elem_bytes(a->out_dtype),
+                   "map_difference: rows too short for %d heads of %d", a->heads, a->vdim);
+    if (v->rows <= 0) return 0;
+    const int waves = 4;
+    PICOLM_REQUIRE(ceil_div(a->heads, waves) <= 65535, "map_difference: %d heads exceed the grid", a->heads);
+    map_difference_kernel<<<dim3(v->rows, ceil_div(a->heads, waves)), waves * WAVE, 0, v->stream>>>((const float*)v->in, v->out, a->out_dtype, a->heads,
+                                                                                                 a->vdim, a->lambda, a->eps, a->mult);
+    PICOLM_LAUNCH_CHECK("map_difference");
+    return 0;
+}

@@ -42,6 +42,42 @@ class PreNormBlock(Block):
         self.ffn.emit(b, self.ffn_norm.emit(b, x), x, after, after_when)
 
 
+class _NoMixer(Mixer):
+    """The mixer of a block that has none: it asks nothing of the cache."""
+
+
+class ParallelBlock(Block):
+    """Mixer and feed-forward as two branches of the same rows, each behind a norm of its own:
+        x <- x + mixer(norm1(x)) + ffn(norm2(x))
+    A block without a feed-forward is x <- x + mixer(norm1(x)).  The second norm is taken before
+    the mixer's output joins x; the two branches then add to x one after the other."""
+    graph_safe = True      # launches depend on device memory only
+
+    def __init__(self, mixer_norm: Norm, mixer: Mixer, ffn_norm: Norm | None, ffn: FeedForward | None):
+        if (ffn is None) != (ffn_norm is None):
+            raise ValueError("a feed-forward and its norm come together")
+        self.mixer_norm, self.mixer, self.ffn_norm, self.ffn = mixer_norm, mixer, ffn_norm, ffn
+
+    def children(self):
+        return [p for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn) if p is not None]
+
+    def first_norm(self):
+        return self.mixer_norm
+
+    def emit(self, b, x: int, after=None, after_when: int = 0) -> None:
+        from ..engine.program import Rows
+        src = self.mixer_norm.emit(b, x)
+        if self.ffn is None:
+            self.mixer.emit(b, src, x, after, after_when)
+            return
+        second = self.ffn_norm.emit(b, x)
+        if second.norm is not None:         # rows of their own: the first norm's place is in use until the mixer has read it
+            second = Rows(b.buffer("norm.out.second", self.ffn_norm.size, b.dtype), second.norm, second.x)
+        held = Rows(b.materialize(second))
+        self.mixer.emit(b, src, x, None, 0)
+        self.ffn.emit(b, held, x, after, after_when)
+
+
 class _WithRowState(Mixer):
     """A mixer as the cache sees it when its block keeps `row_floats` floats of its own per
     sequence in front of the mixer's state: one state entry holds both."""
@@ -156,8 +192,37 @@ class PostNormBlock(Block):
             self._join(b, x, branch, plain, 1, self.ffn_norm)
 
 
-class _NoMixer(Mixer):
-    """The mixer of a block that has none: it asks nothing of the cache."""
+
+
+class LoopSum(Block):
+    """What runs before pass `number` over a looped stretch of layers where the pass is entered by
+    sums alone:  x <- x + x0 (every pass but the first) + step[number], with x0 the embedding's
+    output (which the embedding keeps, `TokenEmbedding(keeps_output=True)`) and step [passes, D]."""
+    graph_safe = True      # launches depend on device memory only
+
+    def __init__(self, step_name: str, hidden_size: int, passes: int, number: int):
+        if not 0 <= number < passes:
+            raise ValueError(f"pass {number} of {passes}")
+        self.D, self.passes, self.number = hidden_size, passes, number
+        self.step_name = step_name
+        self.mixer = _NoMixer()
+        self.step = None
+
+    def tensor_specs(self):
+        from ..weights import TensorSpec
+        return [TensorSpec(self.step_name, (self.passes, self.D))]
+
+    def load(self, fetch, runtime) -> None:
+        import torch
+        self.step = fetch.get(self.step_name).to(torch.float32).contiguous()
+
+    def emit(self, b, x: int, after=None, after_when: int = 0) -> None:
+        import torch
+        from .calls import AddRowsArgs, emit_library_call
+        if self.step is None:
+            raise ValueError(f"loop entry {self.step_name} has no weights loaded")
+        first = b.buffer("embed.out", self.D, torch.float32) if self.number > 0 else -1
+        emit_library_call(b, "add_rows", AddRowsArgs(b._ptr(self.step[self.number]), self.D), x, inp=first)
 
 
 class LoopEntry(Block):

@@ -16,7 +16,9 @@ class SinkAttentionArgs(Structure):
     _fields_ = [("n_heads", c_int32), ("n_kv_heads", c_int32), ("head_dim", c_int32), ("v_head_dim", c_int32),
                 ("in_stride", c_int32), ("q_off", c_int32), ("k_off", c_int32), ("v_off", c_int32), ("gate_off", c_int32),
                 ("scale", c_float), ("eps", c_float),
-                ("q_norm", c_void_p), ("k_norm", c_void_p), ("bias", c_void_p), ("bias_rows", c_int32), ("sink", c_void_p), ("window", c_int32)]
+                ("q_norm", c_void_p), ("k_norm", c_void_p), ("bias", c_void_p), ("bias_rows", c_int32), ("sink", c_void_p), ("window", c_int32),
+                ("chunk", c_int32), ("maps", c_int32), ("out_float", c_int32), ("unit_qk", c_int32), ("in_bias", c_void_p),
+                ("cos_table", c_void_p), ("sin_table", c_void_p), ("table_positions", c_int32), ("rot_dims", c_int32), ("rot_half", c_int32)]
 
 
 class ShortConvArgs(Structure):
@@ -95,7 +97,8 @@ class RouteTopArgs(Structure):
 
 class RoutedExpertsArgs(Structure):
     _fields_ = [("gate", c_void_p), ("up", c_void_p), ("down", c_void_p), ("weight_dt", c_int32), ("experts", c_int32),
-                ("top", c_int32), ("width", c_int32), ("ff", c_int32), ("adds", c_int32), ("identity", c_int32)]
+                ("top", c_int32), ("width", c_int32), ("ff", c_int32), ("adds", c_int32), ("identity", c_int32),
+                ("act", c_int32), ("limit", c_float), ("alpha", c_float), ("weight_on_input", c_int32)]
 
 
 class LayerNormArgs(Structure):
@@ -112,11 +115,20 @@ class RotateHeadsArgs(Structure):
                 ("norm_out_off", c_int32), ("norm_eps", c_float)]
 
 
+class AddRowsArgs(Structure):
+    _fields_ = [("vec", c_void_p), ("width", c_int32)]
+
+
+class MapDifferenceArgs(Structure):
+    _fields_ = [("heads", c_int32), ("vdim", c_int32), ("out_dtype", c_int32), ("lam", c_float), ("eps", c_float), ("mult", c_float)]
+
+
 GATE_NONE, GATE_SILU, GATE_SIGMOID = 0, 1, 2
 DECAY_PER_ROW, DECAY_EXPONENTIAL = 1, 2
 DECAY_SCAN_MAX_KEY_DIM = 256
 MAP_RELU_SQUARED, MAP_SOFTCAP, MAP_SCALE = 1, 2, 3
-SCORE_PICKED_SOFTMAX, SCORE_SOFTMAX_ALL = 0, 1
+SCORE_PICKED_SOFTMAX, SCORE_SOFTMAX_ALL, SCORE_SIGMOID = 0, 1, 2
+EXPERT_SILU_GATED, EXPERT_CLAMPED = 0, 1
 RULE_OUTER_PRODUCT, RULE_DELTA = 0, 1
 STATE_SCAN_MAX_KEY_DIM = 256
 SHORT_CONV_MAX_TAPS = 16

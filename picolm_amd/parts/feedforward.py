@@ -80,13 +80,23 @@ class RoutedExperts(FeedForward):
     output.  The router's logits, the picks and their weights are float; only the picked experts'
     weights are read."""
     graph_safe = True      # launches depend on device memory only
-    SCORINGS = {"picked_softmax": 0, "softmax_all": 1}
+    SCORINGS = {"picked_softmax": 0, "softmax_all": 1, "sigmoid": 2}
+    ACTIVATIONS = {"silu_gated": 0, "clamped": 1}
 
     def __init__(self, prefix: str, hidden_size: int, n_experts: int, top: int, expert_size: int, shared_size: int = 0,
                  names=("gate", "up", "down"), scoring: str = "picked_softmax", identity: int = 0, weight_scale: float = 1.0,
-                 bias_name: str = "router.b", shared_gate: str | None = None):
+                 bias_name: str | None = "router.b", shared_gate: str | None = None, activation: str = "silu_gated",
+                 limit: float = 0.0, alpha: float = 1.0, weight_on_input: bool = False):
+        """`bias_name` None: the router has no bias tensor."""
         if scoring not in self.SCORINGS:
             raise ValueError(f"scoring '{scoring}': known are {', '.join(self.SCORINGS)}")
+        if activation not in self.ACTIVATIONS:
+            raise ValueError(f"activation '{activation}': known are {', '.join(self.ACTIVATIONS)}")
+        if activation == "clamped" and not limit > 0:
+            raise ValueError(f"the clamped activation needs a positive limit, got {limit}")
+        if weight_on_input and identity:
+            raise ValueError("weights on the experts' input and router outputs that give the input back do not go together")
+        self.activation, self.limit, self.alpha, self.weight_on_input = activation, float(limit), float(alpha), bool(weight_on_input)
         if n_experts < 1 or identity < 0 or not 1 <= top <= n_experts + identity:
             raise ValueError(f"{top} picks among {n_experts} experts and {identity} that give their input back")
         if shared_gate and not shared_size:
@@ -111,7 +121,7 @@ class RoutedExperts(FeedForward):
 
     def tensor_specs(self):
         from ..weights import TensorSpec
-        specs = [TensorSpec(self.prefix + self.bias_name, (self.outputs,), init="zeros")]
+        specs = [TensorSpec(self.prefix + self.bias_name, (self.outputs,), init="zeros")] if self.bias_name else []
         for e in range(self.E):
             p = f"{self.prefix}e{e}."
             specs += [TensorSpec(p + self.names[0], (self.F, self.D)), TensorSpec(p + self.names[1], (self.F, self.D)),
@@ -127,7 +137,7 @@ class RoutedExperts(FeedForward):
                 ws = [w.to(torch.float32) for w in ws]
             return torch.stack(ws, dim=0).contiguous()
         self.gate, self.up, self.down = (stacked(n) for n in self.names)
-        self.router_bias = fetch.get(self.prefix + self.bias_name).to(torch.float32).contiguous()
+        self.router_bias = fetch.get(self.prefix + self.bias_name).to(torch.float32).contiguous() if self.bias_name else None
 
     def emit(self, b, src, x: int, out_norm=None, out_norm_when: int = 0, accumulate: bool = True) -> None:
         """x (+)= the picked experts' weighted sum (+ the shared expert) for the rows h of `src`."""
@@ -157,7 +167,8 @@ class RoutedExperts(FeedForward):
             written = True
         hidden = b.buffer("moe.hidden", self.top * self.F, torch.float32)
         args = RoutedExpertsArgs(b._ptr(self.gate), b._ptr(self.up), b._ptr(self.down), _DT[self.gate.dtype], self.E, self.top, self.D,
-                                 self.F, int(written), self.identity)
+                                 self.F, int(written), self.identity, self.ACTIVATIONS[self.activation], self.limit, self.alpha,
+                                 int(self.weight_on_input))
         pair_out = b.buffer("moe.pairs", self.top * self.D, torch.float32)
         plan = b.buffer("moe.plan", self.top + self.E + 1, torch.float32)
         emit_library_call(b, "routed_experts", args, x, inp=h, extra=[picks, hidden, pair_out, plan])
