@@ -192,7 +192,7 @@ class KekelixConfig:
             raise ConfigError("norm.eps: must be positive")
         if self.torch_dtype not in ("bfloat16", "float32", "float16"):
             raise ConfigError(f"torch_dtype: '{self.torch_dtype}' is not one of bfloat16, float32, float16")
-        if self.loop is not None and not 0 <= self.loop.start < self.loop.stop <= len(self.layers):
+        if self.loop is not None and not 0 <= self.loop.start <= self.loop.stop <= len(self.layers):
             raise ConfigError(f"loop: layers {self.loop.start} .. {self.loop.stop - 1} are not a stretch of the {len(self.layers)} layers")
         for e in self.eos_token_ids:
             if not 0 <= e < self.vocab:

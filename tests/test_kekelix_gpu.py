@@ -1,0 +1,529 @@
+"""Kekelix in the engine against the plain model of tests/plain/kekelix_plain.py: every mechanism
+alone, prompts against token-by-token decoding, prompts cut into portions, batches of unequal
+requests, slots and pages that are used again, one key that the asking token's attention rests on
+far back, at page borders, at the first places and just inside and just outside a stretch of
+positions, in prompts and decoded, long decoding through recorded steps, and greedy generation
+through the entry points.
+
+The configurations are those of tests/kekelix_tiny.py; the plain model computes a whole sequence
+from scratch in double precision, so every schedule has one truth: the function of the sequence."""
+import copy
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import kekelix_tiny as kt
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = ["float32", "bfloat16"]
+
+
+def tokens_for(cfg, n, seed):
+    rng = np.random.default_rng(seed)
+    return [int(t) for t in rng.integers(0, cfg["vocab"], size=n)]
+
+
+_MODELS, _TRUTH = {}, {}
+
+
+def model_of(which, dtype, seed=0):
+    key = (which, dtype, seed)
+    if key not in _MODELS:
+        cfg = kt.CONFIGS[which]
+        w = kt.make_weights(cfg, seed)
+        _MODELS[key] = (cfg, w, kt.load(cfg, w, dtype))
+    return _MODELS[key]
+
+
+def truth_of(which, seed, tokens):
+    key = (which, seed, tuple(tokens))
+    if key not in _TRUTH:
+        cfg = kt.CONFIGS[which]
+        _TRUTH[key] = kt.Truth(cfg, kt.make_weights(cfg, seed), tokens)
+    return _TRUTH[key]
+
+
+def new_session(model, max_tokens=4096, **kw):
+    from picolm_amd.engine import Session
+    return Session(model, max_tokens=max_tokens, **kw)
+
+
+def run_whole(session, tokens):
+    [slot] = session.begin(1)
+    got = session.step([slot], [tokens], [list(range(len(tokens)))]).double().cpu().numpy()
+    session.release([slot])
+    return got
+
+
+# ------------------------------------------------------------------------------ each mechanism alone
+def one_layer(mixer, mlp=None, width=48, **kw):
+    return kt.config(61, width, [kt.layer(mixer, mlp)], **kw)
+
+
+_Y = kt.yarn(4.0, 64, 8.0, 2.0)
+_PLAIN_MIXER = kt.sinked(2, 1, 12, 10, 0.3, 8)
+ALONE = {
+    "two maps a head": one_layer(kt.difference(4, 2, 12, 20, 0.3, 0.35)),
+    "two maps a head, a KV head a head": one_layer(kt.difference(3, 3, 10, 6, 0.4, 0.8)),
+    "two maps a head, one head": one_layer(kt.difference(1, 1, 5, 7, 0.5, 0.05)),
+    "two maps, cached keys of 64 and values of 96": one_layer(kt.difference(8, 2, 32, 96, 0.2, 0.3), width=64),       # the matrix-core kernel in bfloat16
+    "two maps, cached keys of 128 and values of 64": one_layer(kt.difference(4, 4, 64, 64, 0.15, 0.5), width=64),
+    "two maps, cached keys of 320": one_layer(kt.difference(2, 1, 160, 24, 0.1, 0.3), width=64),                      # beyond what a thread's registers hold of a key
+    "biases, a part turned, one more in the denominator": one_layer(kt.sinked(6, 2, 20, 12, 0.25, 8, 500.0)),
+    "the whole head turned": one_layer(kt.sinked(3, 1, 12, 20, 0.3, 12, 100.0)),
+    "two entries turned": one_layer(kt.sinked(2, 2, 14, 6, 0.4, 2, 2.0, kt.yarn(2.0, 8, 4.0, 1.0))),
+    "scaled rotation": one_layer(kt.sinked(3, 1, 16, 20, 0.4, 16, 500.0, _Y)),                                        # a ramp from the first pair on
+    "scaled rotation whose ramp starts later": one_layer(kt.sinked(3, 3, 16, 20, 0.4, 16, 500.0, kt.yarn(4.0, 80, 1.0, 0.25))),
+    "scaled rotation whose ramp is one pair wide": one_layer(kt.sinked(2, 1, 12, 6, 0.4, 12, 30.0, kt.yarn(16.0, 40, 2.0, 1.9))),
+    "biases, keys of 96 and values of 64": one_layer(kt.sinked(4, 2, 96, 64, 0.1, 32, 1000.0, _Y), width=64),
+    "biases, keys of 128 and values of 128, forty heads": one_layer(kt.sinked(40, 8, 128, 128, 0.09, 128), width=64),
+    "stretches of 5": one_layer(kt.chunked(3, 1, 12, 0.4, 8, 5)),
+    "stretches of one": one_layer(kt.chunked(2, 1, 12, 0.4, 8, 1)),
+    "stretches of a page": one_layer(kt.chunked(2, 2, 12, 0.4, 12, 64)),
+    "stretches of 33": one_layer(kt.chunked(4, 2, 20, 0.3, 4, 33, 50.0)),
+    "stretches longer than the sequence": one_layer(kt.chunked(2, 1, 12, 0.4, 8, 500)),
+    "stretches of 50, keys of 64": one_layer(kt.chunked(4, 2, 64, 0.2, 32, 50), width=64),
+    "stretches of 65, keys of 96": one_layer(kt.chunked(2, 1, 96, 0.15, 96, 65), width=64),
+    "stretches of 31, keys of 128, twenty heads": one_layer(kt.chunked(20, 4, 128, 0.12, 64, 31), width=64),
+    "stretches of 40, keys of 288": one_layer(kt.chunked(2, 1, 288, 0.1, 32, 40), width=64),
+    "one head of 5": one_layer(kt.chunked(1, 1, 5, 0.6, 4, 9)),
+    "routed experts": one_layer(_PLAIN_MIXER, kt.moe(6, 2, 24, 0.9)),
+    "routed experts, one pick": one_layer(_PLAIN_MIXER, kt.moe(5, 1, 36, 0.5)),
+    "routed experts, one expert": one_layer(_PLAIN_MIXER, kt.moe(1, 1, 20, 1.0)),
+    "routed experts, every expert picked": one_layer(_PLAIN_MIXER, kt.moe(3, 3, 20, 2.0)),
+    "routed experts, a limit that never binds": one_layer(_PLAIN_MIXER, kt.moe(4, 2, 24, 100.0)),
+    "routed experts, a limit that mostly binds": one_layer(_PLAIN_MIXER, kt.moe(4, 2, 24, 0.1)),
+    # in bfloat16 a prompt of 64 rows and more sorts its picks by expert for the matrix cores
+    "routed experts, widths in multiples of 16": one_layer(_PLAIN_MIXER, kt.moe(6, 2, 32, 1.5)),
+    "routed experts, more experts than rows a tile": one_layer(_PLAIN_MIXER, kt.moe(40, 3, 48, 1.0)),
+    "routed experts, widths that are no multiples of 8": one_layer(kt.chunked(1, 1, 9, 0.4, 6, 30), kt.moe(4, 2, 13, 0.8), width=45),
+    "a loop of one pass": kt.config(61, 48, [kt.layer(_PLAIN_MIXER, kt.moe(3, 1, 8, 1.0))], loop=(0, 1, 1)),
+    "a loop of four passes over one layer": kt.config(61, 48, [kt.layer(_PLAIN_MIXER, None)], loop=(0, 1, 4)),
+    "a loop that starts behind the first layer and ends before the last": kt.config(61, 48, [
+        kt.layer(kt.difference(2, 1, 6, 8, 0.4, 0.3), None), kt.layer(kt.chunked(2, 1, 12, 0.4, 8, 7), None), kt.layer(_PLAIN_MIXER, None)],
+        loop=(1, 2, 2)),
+    "eps": one_layer(kt.difference(2, 1, 12, 10, 0.3, 0.4), kt.moe(3, 2, 24, 1.0), eps=1e-2),
+}
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("what", list(ALONE))
+def test_each_mechanism_alone(what, dtype):
+    cfg = ALONE[what]
+    w = kt.make_weights(cfg, 11)
+    tokens = tokens_for(cfg, 70, 3)            # past a page's end
+    want = kt.Truth(cfg, w, tokens)
+    s = new_session(kt.load(cfg, w, dtype), 256)
+    assert kt.near(run_whole(s, tokens), want, slice(None), dtype)
+    # and the same decoded token by token
+    [slot] = s.begin(1)
+    for i, t in enumerate(tokens):
+        got = s.step([slot], [[t]]).double().cpu().numpy()
+        assert kt.near(got, want, i, dtype), (what, "token", i)
+    s.release([slot])
+
+
+# ------------------------------------------------------------------------------ prompts, decoding, portions
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("which", ["A", "B", "C"])
+def test_prompt_decoding_and_portions(which, dtype):
+    cfg, w, model = model_of(which, dtype)
+    tokens = tokens_for(cfg, 150, 1)
+    want = truth_of(which, 0, tokens)
+    s = new_session(model, 1024)
+    assert kt.near(run_whole(s, tokens), want, slice(None), dtype)
+    # most of it at once, the rest one by one (past the page border at 128, and past the ends of stretches)
+    [slot] = s.begin(1)
+    got = s.step([slot], [tokens[:101]], [[0, 1, 2, 63, 64, 100]]).double().cpu().numpy()
+    assert kt.near(got, want, [0, 1, 2, 63, 64, 100], dtype)
+    for i in range(101, 150):
+        got = s.step([slot], [[tokens[i]]]).double().cpu().numpy()
+        assert kt.near(got, want, i, dtype), ("decoded", i)
+    s.release([slot])
+    # portions of several sizes, down to two tokens and one, every row wanted
+    for sizes in ([2, 2, 3, 57, 1, 64, 21], [64, 64, 22], [1, 1, 2, 146], [149, 1], [36, 37, 38, 39]):
+        assert sum(sizes) == 150
+        [slot] = s.begin(1)
+        at = 0
+        for n in sizes:
+            got = s.step([slot], [tokens[at:at + n]], [list(range(n))]).double().cpu().numpy()
+            assert kt.near(got, want, slice(at, at + n), dtype), (sizes, "portion at", at)
+            at += n
+        s.release([slot])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_portions_equal_the_whole_prompt_beyond_rounding(dtype):
+    """How a prompt is cut does not show in the logits: against each other, not only against the
+    plain model, and much closer than the limit that bfloat16 needs there."""
+    cfg, w, model = model_of("A", dtype)
+    tokens = tokens_for(cfg, 131, 5)
+    s = new_session(model, 1024)
+    whole = run_whole(s, tokens)
+    [slot] = s.begin(1)
+    parts, at = [], 0
+    for n in (2, 63, 2, 61, 3):
+        parts.append(s.step([slot], [tokens[at:at + n]], [list(range(n))]).double().cpu().numpy())
+        at += n
+    s.release([slot])
+    assert kt.distance(np.concatenate(parts), whole) <= (1e-5 if dtype == "float32" else 0.03)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("which", ["A", "B"])
+def test_a_long_prompt(which, dtype):
+    """Several pages and several tiles of queries, stretches that end inside pages; whole, in two long
+    portions, and beside short requests in a batch, then decoded on."""
+    cfg, w, model = model_of(which, dtype)
+    tokens = tokens_for(cfg, 405, 8)
+    want = truth_of(which, 0, tokens)
+    s = new_session(model, 2048)
+    assert kt.near(run_whole(s, tokens[:401]), want, slice(0, 401), dtype)
+    [slot] = s.begin(1)
+    rows = [0, 63, 64, 127, 128, 199]
+    got = s.step([slot], [tokens[:200]], [rows]).double().cpu().numpy()
+    assert kt.near(got, want, rows, dtype)
+    got = s.step([slot], [tokens[200:401]], [list(range(201))]).double().cpu().numpy()
+    assert kt.near(got, want, slice(200, 401), dtype)
+    for i in range(401, 405):
+        got = s.step([slot], [[tokens[i]]]).double().cpu().numpy()
+        assert kt.near(got, want, i, dtype), ("decoded", i)
+    s.release([slot])
+    others = [tokens_for(cfg, n, 30 + n) for n in (10, 257)]
+    slots = s.begin(3)
+    got = s.step(slots, [tokens[:400]] + others).double().cpu().numpy()
+    assert kt.near(got[0], want, 399, dtype)
+    for i, q in enumerate(others):
+        assert kt.near(got[1 + i], truth_of(which, 0, q), len(q) - 1, dtype), ("beside the long one", i)
+    got = s.step(slots[:1], [[tokens[400]]]).double().cpu().numpy()
+    assert kt.near(got, want, 400, dtype)
+    s.release(slots)
+
+
+# ------------------------------------------------------------------------------ batches
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("which", ["A", "C"])
+def test_a_batch_of_unequal_requests_equals_each_alone(which, dtype):
+    cfg, w, model = model_of(which, dtype)
+    lens, n_dec = [1, 2, 65, 37, 64, 130], 5
+    seqs = [tokens_for(cfg, n + n_dec, 20 + i) for i, n in enumerate(lens)]
+    truth = [truth_of(which, 0, q) for q in seqs]
+    s = new_session(model, 2048)
+    slots = s.begin(len(seqs))
+    got = s.step(slots, [q[:n] for q, n in zip(seqs, lens)], [list(range(n)) for n in lens]).double().cpu().numpy()
+    at = 0
+    for i, n in enumerate(lens):
+        assert kt.near(got[at:at + n], truth[i], slice(0, n), dtype), ("prompt", i)
+        at += n
+    # and against each alone, much closer than the plain model is in bfloat16: what else is in the batch does not show
+    alone = new_session(model, 512)
+    at = 0
+    for i, n in enumerate(lens):
+        assert kt.distance(got[at:at + n], run_whole(alone, seqs[i][:n])) <= (1e-5 if dtype == "float32" else 0.03), ("alone", i)
+        at += n
+    # the shorter ones end earlier: after two steps the first two leave the batch
+    live = list(range(len(seqs)))
+    for j in range(n_dec):
+        if j == 2:
+            s.release([slots[0], slots[1]])
+            live = live[2:]
+        got = s.step([slots[i] for i in live], [[seqs[i][lens[i] + j]] for i in live]).double().cpu().numpy()
+        for row, i in enumerate(live):
+            assert kt.near(got[row], truth[i], lens[i] + j, dtype), ("step", j, "sequence", i)
+    s.release([slots[i] for i in live])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_slots_and_pages_that_are_used_again(dtype):
+    """A page's old keys are not seen: sequences run one after another through a session that has
+    room for little more than one of them."""
+    cfg, w, model = model_of("A", dtype)
+    s = new_session(model, 256, n_slots=2)
+    for k, n in enumerate([130, 5, 70, 130, 1, 64]):
+        tokens = tokens_for(cfg, n, 40 + k)
+        want = truth_of("A", 0, tokens)
+        [slot] = s.begin(1)
+        cut = max(1, n - 3)
+        rows = [0, cut - 1]
+        got = s.step([slot], [tokens[:cut]], [rows]).double().cpu().numpy()
+        assert kt.near(got, want, rows, dtype), ("prompt", k)
+        for i in range(cut, n):
+            got = s.step([slot], [[tokens[i]]]).double().cpu().numpy()
+            assert kt.near(got, want, i, dtype), ("sequence", k, "token", i)
+        s.release([slot])
+    # two sequences that swap slots between uses
+    a, b = tokens_for(cfg, 40, 90), tokens_for(cfg, 66, 91)
+    for order in ((a, b), (b, a)):
+        slots = s.begin(2)
+        got = s.step(slots, list(order)).double().cpu().numpy()
+        for i, q in enumerate(order):
+            assert kt.near(got[i], truth_of("A", 0, q), len(q) - 1, dtype)
+        s.release(slots)
+
+
+# ------------------------------------------------------------------------------ far keys, page borders, stretches' edges
+def lookup_model(kind, dim=32, size=0, width=64):
+    """One layer whose attention looks a token's partner up.  Token t + 700 has the first half of
+    token t's embedding.  Keys read the first half of the width (strongly) and queries are the keys'
+    rows, so the score of two tokens with the same first half is as high as a token's with itself
+    and far above the chance products of hundreds of other keys; what the partner contributes
+    differs from the asking token's own contribution through the second half of the width (the
+    values read it; where the values are the keys, the keys read it weakly).  Few entries are
+    turned, so that the position hardly weakens the match.  So the asking token's output rests on
+    its partner wherever the partner stands, if it is seen."""
+    half, heads = width // 2, 2
+    scale = 30.0 / dim
+    if kind == "attention":
+        mixer = kt.difference(heads, 1, dim, 16, scale, 0.3)
+    elif kind == "attention_2":
+        mixer = kt.sinked(heads, 1, dim, 16, scale, 4, 10000.0, kt.yarn(4.0, 64, 8.0, 2.0))
+    else:
+        mixer = kt.chunked(heads, 1, dim, scale, 4, size, 10000.0)
+    cfg = kt.config(1400, width, [kt.layer(mixer, None)])
+    w = kt.make_weights(cfg, 5)
+    w["embed"][700:, :half] = w["embed"][:700, :half]
+    w["l0.norm1"] = torch.zeros(width, dtype=torch.bfloat16)
+    p = "l0.mix."
+    gen = torch.Generator().manual_seed(2)
+    keys = torch.randn(dim, width, generator=gen, dtype=torch.float64) / half ** 0.5
+    keys[:, half:] = 0
+    if kind == "attention":
+        # map 1 looks the partner up; map 2's scores are small, so that it spreads over all keys
+        k = torch.cat([keys, 0.05 * torch.randn(dim, width, generator=gen, dtype=torch.float64)])
+        w[p + "k"] = k.to(torch.bfloat16)
+        w[p + "q"] = torch.cat([k] * heads).to(torch.bfloat16)
+    elif kind == "attention_2":
+        w[p + "k"] = keys.to(torch.bfloat16)
+        w[p + "q"] = torch.cat([keys] * heads).to(torch.bfloat16)
+        for n in ("q.b", "k.b", "v.b"):
+            w[p + n] = (0.1 * w[p + n].double()).to(torch.bfloat16)
+    else:
+        k = keys.clone()
+        k[:, half:] = 0.3 * torch.randn(dim, half, generator=gen, dtype=torch.float64) / half ** 0.5     # the values are the keys
+        w[p + "k"] = k.to(torch.bfloat16)
+        w[p + "q"] = torch.cat([keys] * heads).to(torch.bfloat16)
+    if kind != "attention_3":
+        w[p + "v"][:, :half] = 0
+        w[p + "v"] = (4.0 * w[p + "v"].double()).to(torch.bfloat16)
+    w[p + "o"] = (16.0 * w[p + "o"].double()).to(torch.bfloat16)          # the branch outweighs the rows it is added to
+    return cfg, w
+
+
+def distinct_tokens(n, needle_at, vocab, seed):
+    """n unrelated tokens, except that the last one's partner stands at `needle_at`."""
+    rng = np.random.default_rng(seed)
+    tokens = [int(t) for t in rng.permutation(vocab // 2)[:n]]
+    tokens[needle_at] = tokens[-1] + vocab // 2
+    return tokens
+
+
+def without_the_partner(tokens, needle_at, vocab):
+    other = list(tokens)
+    other[needle_at] = next(t for t in range(vocab // 2) if t not in tokens)
+    return other
+
+
+_FAR = {}
+
+
+def asking_sequence(key, cfg, w, n, needle_at, seed, seen=True):
+    """n tokens whose last one's partner stands at `needle_at`, the plain model's logits of the last
+    token, and a check that the test can tell: with the partner replaced by an unrelated token the
+    logits differ by far more than rounding if the partner is seen (tokens are drawn again until
+    they do), and not at all if it lies in an earlier stretch (while they would if one stretch
+    covered the sequence)."""
+    if key in _FAR:
+        return _FAR[key]
+    while True:
+        tokens = distinct_tokens(n, needle_at, cfg["vocab"], seed)
+        other = without_the_partner(tokens, needle_at, cfg["vocab"])
+        want, missed = kt.plain_logits(cfg, w, tokens)[-1], kt.plain_logits(cfg, w, other)[-1]
+        if not seen:
+            assert kt.distance(missed, want) < 1e-9, "the key must not count"
+            whole = copy.deepcopy(cfg)
+            whole["layers"][0]["mixer"]["mask"]["size"] = n
+            counts = kt.distance(kt.plain_logits(whole, w, other)[-1], kt.plain_logits(whole, w, tokens)[-1])
+        else:
+            counts = kt.distance(missed, want) if needle_at != n - 1 else 1.0
+        if counts > 0.2:
+            _FAR[key] = (tokens, want)
+            return _FAR[key]
+        seed += 1000
+
+
+def ask_in_a_prompt_and_decoded(s, tokens, want, dtype, what):
+    [slot] = s.begin(1)
+    got = s.step([slot], [tokens]).double().cpu().numpy()
+    assert kt.distance(got, want) <= kt.LIMIT[dtype], ("prompt",) + what
+    s.release([slot])
+    [slot] = s.begin(1)
+    s.step([slot], [tokens[:-1]], [[]])
+    got = s.step([slot], [tokens[-1:]]).double().cpu().numpy()
+    assert kt.distance(got, want) <= kt.LIMIT[dtype], ("decoded",) + what
+    s.release([slot])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("kind,dim", [("attention", 20), ("attention", 32), ("attention_2", 24), ("attention_2", 64), ("attention_3", 40),
+                                      ("attention_3", 64)])
+def test_one_far_key_among_hundreds(kind, dim, dtype):
+    """The asking token is the last; the key it asks for lies hundreds back, at the first places of
+    the sequence, and just before and after page borders.  Both in a prompt and decoded.  (Cached
+    keys of 64 go through the matrix-core kernel in bfloat16, the others through the vector ALU.)"""
+    cfg, w = lookup_model(kind, dim, size=1000)
+    s = new_session(kt.load(cfg, w, dtype), 2048)
+    n = 500
+    for needle_at in (0, 1, 63, 64, 65, 128, 383, 498):
+        tokens, want = asking_sequence((kind, dim, needle_at), cfg, w, n, needle_at, needle_at)
+        ask_in_a_prompt_and_decoded(s, tokens, want, dtype, (needle_at,))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("size,dim", [(70, 40), (64, 40), (129, 40), (2, 40), (33, 64), (100, 64), (200, 64)])
+def test_a_key_just_inside_and_just_outside_a_stretch(size, dim, dtype):
+    """The partner of the last token stands at the first place of the last token's stretch and at
+    the place before it: seen, the logits rest on it; not seen, they are what they are without it.
+    The asking token is the second of its stretch, the last of it, and somewhere between."""
+    cfg, w = lookup_model("attention_3", dim, size)
+    s = new_session(kt.load(cfg, w, dtype), 1024)
+    for n in {2 * size + 2, 3 * size, 4 * size + max(2, size // 2)}:
+        first = (n - 1) // size * size
+        if first == n - 1 or n > 690:          # (the vocabulary has 700 unrelated tokens)
+            continue
+        for needle_at, seen in ((first, True), (first - 1, False)):
+            tokens, want = asking_sequence((size, dim, n, needle_at), cfg, w, n, needle_at, n + needle_at, seen)
+            ask_in_a_prompt_and_decoded(s, tokens, want, dtype, (n, needle_at))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("size,dim", [(70, 40), (37, 64)])
+def test_a_stretch_ends_among_decoded_tokens(size, dim, dtype):
+    """A short prompt, then single tokens until the asking one, in a batch with a sequence that
+    started elsewhere: the partner was decoded as the first token of the asking token's stretch
+    (seen) or as the last of the stretch before (not seen), or stood in the prompt, stretches back."""
+    cfg, w = lookup_model("attention_3", dim, size)
+    s = new_session(kt.load(cfg, w, dtype), 1024)
+    beside = distinct_tokens(400, 3, cfg["vocab"], 77)
+    n = 2 * size + 9
+    for needle_at, seen in ((2 * size, True), (2 * size - 1, False), (5, False)):
+        tokens, want = asking_sequence(("decoded", size, dim, needle_at), cfg, w, n, needle_at, needle_at, seen)
+        slots = s.begin(2)
+        s.step(slots, [tokens[:8], beside[:400 - (n - 8)]], [[], []])
+        for i in range(8, n):
+            got = s.step(slots, [[tokens[i]], [beside[400 - n + i]]]).double().cpu().numpy()
+        assert kt.distance(got[0], want) <= kt.LIMIT[dtype], (needle_at, seen)
+        s.release(slots)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_the_first_tokens_of_a_sequence(dtype):
+    """Sequences of one, two and three tokens, alone and in one batch; stretches of one and two."""
+    cfg, w, model = model_of("C", dtype)
+    s = new_session(model, 512)
+    seqs = [tokens_for(cfg, n, 60 + n) for n in (1, 2, 3, 1)]
+    for q in seqs:
+        assert kt.near(run_whole(s, q), truth_of("C", 0, q), slice(None), dtype)
+    slots = s.begin(len(seqs))
+    got = s.step(slots, seqs).double().cpu().numpy()
+    for i, q in enumerate(seqs):
+        assert kt.near(got[i], truth_of("C", 0, q), len(q) - 1, dtype)
+    s.release(slots)
+
+
+# ------------------------------------------------------------------------------ long decoding
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("which", ["A", "B"])
+def test_long_decoding_through_recorded_steps(which, dtype):
+    """Three sequences decoded 200 tokens, over page borders and past the ends of stretches; from
+    the second step of a shape on the engine replays its recording."""
+    cfg, w, model = model_of(which, dtype)
+    lens, n_dec = [3, 60, 120], 200
+    seqs = [tokens_for(cfg, n + n_dec, 70 + i) for i, n in enumerate(lens)]
+    truth = [truth_of(which, 0, q) for q in seqs]
+    s = new_session(model, 2048)
+    slots = s.begin(3)
+    s.step(slots, [q[:n] for q, n in zip(seqs, lens)])
+    for j in range(n_dec):
+        got = s.step(slots, [[q[n + j]] for q, n in zip(seqs, lens)]).double().cpu().numpy()
+        for i, n in enumerate(lens):
+            assert kt.near(got[i], truth[i], n + j, dtype), ("step", j, "sequence", i)
+    assert s.recorded_steps() >= 1
+    s.release(slots)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_recorded_and_launched_steps_give_the_same_bits(dtype):
+    cfg, w, model = model_of("A", dtype)
+    seqs = [tokens_for(cfg, n + 12, 170 + i) for i, n in enumerate([5, 70])]
+    rows = {}
+    for graphs in (True, False):
+        s = new_session(model, 1024, graphs=graphs)
+        slots = s.begin(2)
+        s.step(slots, [seqs[0][:5], seqs[1][:70]])
+        rows[graphs] = [s.step(slots, [[seqs[0][5 + j]], [seqs[1][70 + j]]]).cpu().numpy().copy() for j in range(12)]
+        s.release(slots)
+    for a, b in zip(rows[True], rows[False]):
+        assert np.array_equal(a, b)
+
+
+# ------------------------------------------------------------------------------ the entry points
+@pytest.fixture(scope="module")
+def folder_a(tmp_path_factory):
+    cfg = kt.CONFIGS["A"]
+    return kt.write_folder(str(tmp_path_factory.mktemp("kekelix") / "a"), cfg, kt.make_weights(cfg, 0))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_greedy_generation_through_the_entry_point(dtype, folder_a):
+    import picolm_amd
+    cfg = kt.CONFIGS["A"]
+    prompts = [tokens_for(cfg, n, 50 + n) for n in (4, 9, 66)]
+    got = picolm_amd.generate(folder_a, prompts, max_new_tokens=10, stop_ids=(), dtype=dtype)
+    for p, r in zip(prompts, got):
+        assert len(r.tokens) == 10 and r.finish == "length"
+        seq = list(p)
+        for k in range(10):
+            t = truth_of("A", 0, seq)
+            lg = t.logits[-1]
+            top2 = np.sort(lg)[-2:]
+            if top2[1] - top2[0] < 4 * kt.LIMIT[dtype] * lg.std() or t.margins[-kt.AFTER - 1:].min() < kt.CLOSE_CALL[dtype]:
+                break                              # a near tie, or a router's close call: either choice is right
+            assert r.tokens[k] == int(np.argmax(lg)), (k, r.tokens)
+            seq.append(r.tokens[k])
+
+
+def test_trace_replay_and_command_line(folder_a, tmp_path):
+    """bin/trace_run on a folder: a prompt, single tokens and a second request that joins later in a
+    slot that was given back; bin/picolm generates from the same folder."""
+    cfg = kt.CONFIGS["A"]
+    a, b = tokens_for(cfg, 20, 1), tokens_for(cfg, 9, 2)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:17], "want": [0, 16]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": a[17:18], "want": [0]}], "end": []},
+             {"step": 2, "entries": [{"id": "a", "tokens": a[18:19], "want": []}], "end": []},
+             {"step": 3, "entries": [{"id": "a", "tokens": a[19:20], "want": [0]}], "end": ["a"]},
+             {"step": 4, "entries": [{"id": "b", "tokens": b, "want": [8]}], "end": ["b"]}]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = str(tmp_path / "out")
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder_a, "--dtype", "float32", "--out", out,
+                        "--max-tokens", "128"], input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True,
+                       timeout=300)
+    assert r.returncode == 0, r.stderr
+    assert [l for l in r.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(5)]
+    ta, tb = truth_of("A", 0, a), truth_of("A", 0, b)
+    read = lambda i: np.fromfile(os.path.join(out, f"{i}.f32"), dtype="<f4").reshape(-1, cfg["vocab"])
+    assert kt.near(read(0), ta, [0, 16], "float32")
+    assert kt.near(read(1), ta, 17, "float32")
+    assert not os.path.exists(os.path.join(out, "2.f32"))
+    assert kt.near(read(3), ta, 19, "float32")
+    assert kt.near(read(4), tb, 8, "float32")
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "picolm"), folder_a, "-p", " ".join(map(str, b)), "-n", "4", "-t", "0",
+                        "--dtype", "float32"], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr
+    assert len(r.stdout.split()) == 4
+    assert int(r.stdout.split()[0]) == int(np.argmax(tb.logits[-1]))
