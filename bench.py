@@ -271,7 +271,56 @@ def _satedra_rooflines(cfg: dict, T: int, n_seq: int, context: int) -> dict:
     return {"prefill": pre, "decode": dec}
 
 
+def _kekelix_pair(width: int, heads: int, stretch: int, experts: int, top: int, vocab: int, runs: int):
+    """A Kekelix of `runs` layer runs with heads of 128: a layer of two attention maps a head (keys of
+    64 each, so a cached key of 128) that a loop runs twice, a layer whose values are its keys and whose
+    queries see stretches of `stretch` positions, and from four runs on a layer with biases, half of
+    every head turned (YaRN-scaled) and one more in the softmax's denominator; a KV head for four query
+    heads; `experts` experts as wide as the model of which a token uses `top`.  And the Satedra of as
+    many layer runs of the same width, heads, vocabulary, experts and a cached key as long, whose
+    windows are `stretch` keys."""
+    mlp = dict(kind="moe", router=dict(experts=experts, top=top), expert=dict(ff=width, limit=7.0))
+    G = max(heads // 4, 1)
+    kinds = [dict(type="attention", mixer=dict(heads=heads, kv_heads=G, dim=64, vdim=128, scale=64 ** -0.5, diff=0.3), mlp=mlp),
+             dict(type="attention_3", mixer=dict(heads=heads, kv_heads=G, dim=128, vdim=128, scale=128 ** -0.5,
+                                                 rot=dict(base=250000.0, dims=64), mask=dict(size=stretch)), mlp=mlp),
+             dict(type="attention_2", mixer=dict(heads=heads, kv_heads=G, dim=128, vdim=128, scale=128 ** -0.5,
+                                                 rot=dict(base=10000.0, dims=64, scaling=dict(factor=8.0, original=4096, fast=32.0, slow=1.0))),
+                  mlp=mlp)]
+    layers = kinds[:runs - 1]
+    kek = dict(architecture="Kekelix", vocab=vocab, width=width, norm=dict(eps=1e-6), layers=layers, loop=dict(start=0, stop=1, times=2))
+    sat, _ = _satedra_pair(width, heads, 96, 32, stretch, experts, top, vocab, runs)
+    return kek, sat
+
+
+def _kekelix_rooflines(cfg: dict, T: int, n_seq: int, context: int) -> dict:
+    """As _satedra_rooflines: the attention over the keys a query sees (both maps of a layer with two,
+    each with keys of its own and the same values) and the picked experts' products at the bf16 matrix
+    peak; in a decode step the keys and values that the new token sees once per sequence and the
+    weights of the experts that the step's tokens can pick at most, at HBM's peak."""
+    mfma, hbm = PEAK_TFLOPS["bf16"] * 1e12, HBM_PEAK_GBS * 1e9
+    names = ("sink_attention", "routed_experts")
+    pre, dec = {k: 0.0 for k in names}, {k: 0.0 for k in names}
+    D, loop = cfg["width"], cfg.get("loop")
+    for i, layer in enumerate(cfg["layers"]):
+        times = loop["times"] if loop and loop["start"] <= i < loop["stop"] else 1
+        m = layer["mixer"]
+        maps = 2 if layer["type"] == "attention" else 1
+        size = (m.get("mask") or {}).get("size", 0) or T + context + 1
+        seen = sum(j % size + 1 for j in range(T))
+        pre["sink_attention"] += times * 2.0 * m["heads"] * maps * (m["dim"] + m["vdim"]) * seen / mfma
+        dec["sink_attention"] += times * n_seq * (context % size + 1) * m["kv_heads"] * (maps * m["dim"] + m["vdim"]) * 2 / hbm
+        mlp = layer.get("mlp")
+        if mlp:
+            E, top, F = mlp["router"]["experts"], mlp["router"]["top"], mlp["expert"]["ff"]
+            pre["routed_experts"] += times * 2.0 * 3 * T * top * D * F / mfma
+            dec["routed_experts"] += times * min(n_seq * top, E) * 3 * D * F * 2 / hbm
+    return {"prefill": pre, "decode": dec}
+
+
 DESIGN_SIZES = {
+    "kekelix": [("width 1024", (1024, 8, 1536, 8, 2, 32000, 4)), ("width 2048", (2048, 16, 1536, 8, 2, 32000, 4)),
+                ("width 4096", (4096, 32, 1536, 16, 2, 128256, 3))],
     "begopel": [("width 1024", (1024, 8, 2, 4096, 32000, 2, 2)), ("width 2048", (2048, 16, 4, 8192, 32000, 2, 0)),
                 ("width 4096", (4096, 32, 8, 14336, 128256, 1, 0))],
     "zarinex": [("width 1024", (1024, 8, 128, 8, 2, 32000, 4)), ("width 2048", (2048, 16, 128, 8, 2, 32000, 4)),
@@ -315,7 +364,7 @@ def _zarinex_rooflines(cfg: dict, T: int, n_seq: int, context: int) -> dict:
 def design_comparison(design: str, T: int, n_seq: int, context: int, steps: int) -> dict:
     """Prefill and decode throughput of `design` at a few sizes that resemble real layers (random
     weights), beside the closest model the library has at equal size (for Begopel the Llama, for
-    Zarinex the Begopel, for Satedra the Zarinex), and the GPU time of one prefill step and one decode step by operation."""
+    Zarinex the Begopel, for Satedra the Zarinex, for Kekelix the Satedra), and the GPU time of one prefill step and one decode step by operation."""
     import torch
 
     from picolm_amd.config import LlamaConfig, resolve
@@ -375,6 +424,14 @@ def design_comparison(design: str, T: int, n_seq: int, context: int, steps: int)
 
     for name, size in DESIGN_SIZES[design]:
         print(f"[bench] {design} {name}", file=sys.stderr, flush=True)
+        if design == "kekelix":
+            kek, sat = _kekelix_pair(*size)
+            a = measure(resolve(kek).parse_config(kek), kek["vocab"])
+            b = measure(resolve(sat).parse_config(sat), sat["vocab"])
+            out["sizes"].append({"size": name, "layer_runs": size[-1], design: a, "satedra": b,
+                                 "fraction_of_roofline": fractions_of(_kekelix_rooflines(kek, T, n_seq, context), a),
+                                 "satedra_fraction_of_roofline": fractions_of(_satedra_rooflines(sat, T, n_seq, context), b)})
+            continue
         if design == "satedra":
             sat, zar = _satedra_pair(*size)
             a = measure(resolve(sat).parse_config(sat), sat["vocab"])
