@@ -74,8 +74,10 @@ class KekelixMixer:
             rot = RotationConfig.from_dict(_object(d, where, "rot"), where + "rot.")
         if kind == "attention_3":
             mask = _integer(_object(d, where, "mask"), where + "mask.", "size")
-        c = KekelixMixer(kind, _integer(d, where, "heads"), _integer(d, where, "kv_heads"), _integer(d, where, "dim"),
-                         _integer(d, where, "vdim"), _number(d, where, "scale"), diff, rot, mask or 0)
+        dim = _integer(d, where, "dim")
+        # where the values are the keys they have the keys' size, whatever `vdim` says
+        c = KekelixMixer(kind, _integer(d, where, "heads"), _integer(d, where, "kv_heads"), dim,
+                         dim if kind == "attention_3" else _integer(d, where, "vdim"), _number(d, where, "scale"), diff, rot, mask or 0)
         if c.heads % c.kv_heads:
             raise ConfigError(f"{where}kv_heads: {c.kv_heads} does not divide heads = {c.heads}")
         key = 2 * c.dim if kind == "attention" else c.dim          # both maps' keys of a token are cached side by side
@@ -87,8 +89,6 @@ class KekelixMixer:
             raise ConfigError(f"{where}scale: must be positive")
         if rot is not None and rot.dims > c.dim:
             raise ConfigError(f"{where}rot.dims: {rot.dims} entries of a head of {c.dim}")
-        if kind == "attention_3" and c.vdim != c.dim:
-            raise ConfigError(f"{where}vdim: {c.vdim} is not dim = {c.dim}, and the values are the keys")
         return c
 
     def to_dict(self) -> dict:

@@ -35,7 +35,7 @@ def test_the_registry_knows_the_name_and_the_configuration_round_trips():
     (("layers", 0, "mixer", "rot", "scaling", "slow"), 0.0, "layers[0].mixer.rot.scaling.slow"),
     (("layers", 1, "mixer", "diff"), None, "layers[1].mixer.diff"), (("layers", 1, "mixer", "dim"), 600, "layers[1].mixer.dim"),
     (("layers", 1, "mixer", "scale"), 0.0, "layers[1].mixer.scale"), (("layers", 2, "mixer", "mask"), None, "layers[2].mixer.mask"),
-    (("layers", 2, "mixer", "mask", "size"), 0, "layers[2].mixer.mask.size"), (("layers", 2, "mixer", "vdim"), 20, "layers[2].mixer.vdim"),
+    (("layers", 2, "mixer", "mask", "size"), 0, "layers[2].mixer.mask.size"),
     (("layers", 0, "mlp", "kind"), "dense", "layers[0].mlp.kind"), (("layers", 0, "mlp", "router", "top"), 9, "layers[0].mlp.router.top"),
     (("layers", 0, "mlp", "expert", "limit"), 0.0, "layers[0].mlp.expert.limit"), (("layers", 0, "mlp", "expert"), None, "layers[0].mlp.expert"),
     (("loop", "stop"), 9, "loop"), (("loop", "times"), 0, "loop.times"),
