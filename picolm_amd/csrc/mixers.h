@@ -297,6 +297,17 @@ typedef struct {
 } picolm_add_rows_args;
 int picolm_call_add_rows(void* user, const picolm_step_view* v);
 
+// Two RMS norms of the same float rows, which share the root: a = x / sqrt(mean(x^2) + eps) * w_a and
+// b = the same times w_b: what a layer needs whose two branches read the same rows, each behind a norm
+// of its own.  in: x float rows [width]; out: a, rows [width] of out_dtype; extra[0]: b, likewise.
+typedef struct {
+    const float* w_a;        // [width]
+    const float* w_b;
+    int32_t width, out_dtype;
+    float eps;
+} picolm_rms_pair_args;
+int picolm_call_rms_pair(void* user, const picolm_step_view* v);
+
 // Two attention maps a head become one: o = a1 - lambda a2, divided by its root mean square over the
 // head's `vdim` values (eps inside the root, no weight), times `mult`.
 //   in: float rows [heads][2][vdim], map m of head h at (2 h + m) vdim; out: rows [heads vdim] of out_dtype.

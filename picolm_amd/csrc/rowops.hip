@@ -595,3 +595,40 @@ extern "C" int picolm_call_map_difference(void* user, const picolm_step_view* v)
     PICOLM_LAUNCH_CHECK("map_difference");
     return 0;
 }
+
+// ---- two norms of the same rows -------------------------------------------------------------------------
+// a workgroup a row: the row is read once for the sum of squares and once more (from cache) for the outputs
+template <typename T>
+__global__ __launch_bounds__(256) void rms_pair_kernel(const float* __restrict__ x, T* __restrict__ a, T* __restrict__ b,
+                                                       const float* __restrict__ w_a, const float* __restrict__ w_b, int W, float eps) {
+    __shared__ float scratch[16];
+    const size_t row = blockIdx.x;
+    const float* xr = x + row * W;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < W; c += blockDim.x) ss += xr[c] * xr[c];
+    ss = block_sum(ss, scratch);
+    const float inv = 1.f / sqrtf(ss / (float)W + eps);
+    for (int c = threadIdx.x; c < W; c += blockDim.x) {
+        const float y = xr[c] * inv;
+        a[row * W + c] = from_f32<T>(y * w_a[c]);
+        b[row * W + c] = from_f32<T>(y * w_b[c]);
+    }
+}
+
+extern "C" int picolm_call_rms_pair(void* user, const picolm_step_view* v) {
+    const picolm_rms_pair_args* a = (const picolm_rms_pair_args*)user;
+    VIEW_REQUIRE("rms_pair", v);
+    PICOLM_REQUIRE(a && a->w_a && a->w_b && a->width > 0 && known_dtype(a->out_dtype) && v->in && v->out && v->extra[0] && v->out != v->extra[0],
+                   "rms_pair: weights or buffers are missing (the two outputs differ)");
+    const int es = elem_bytes(a->out_dtype);
+    PICOLM_REQUIRE(v->in_row_bytes >= a->width * 4 && v->out_row_bytes >= a->width * es && v->extra_row_bytes[0] >= a->width * es,
+                   "rms_pair: rows too short for a width of %d", a->width);
+    if (v->rows <= 0) return 0;
+    if (a->out_dtype == PICOLM_F32)
+        rms_pair_kernel<float><<<v->rows, 256, 0, v->stream>>>((const float*)v->in, (float*)v->out, (float*)v->extra[0], a->w_a, a->w_b, a->width, a->eps);
+    else
+        rms_pair_kernel<bf16_t><<<v->rows, 256, 0, v->stream>>>((const float*)v->in, (bf16_t*)v->out, (bf16_t*)v->extra[0], a->w_a, a->w_b, a->width,
+                                                                a->eps);
+    PICOLM_LAUNCH_CHECK("rms_pair");
+    return 0;
+}

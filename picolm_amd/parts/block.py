@@ -49,8 +49,9 @@ class _NoMixer(Mixer):
 class ParallelBlock(Block):
     """Mixer and feed-forward as two branches of the same rows, each behind a norm of its own:
         x <- x + mixer(norm1(x)) + ffn(norm2(x))
-    A block without a feed-forward is x <- x + mixer(norm1(x)).  The second norm is taken before
-    the mixer's output joins x; the two branches then add to x one after the other."""
+    A block without a feed-forward is x <- x + mixer(norm1(x)).  Both norms are taken before the
+    mixer's output joins x (two RMS norms with one eps in one pass over the rows, `rms_pair`: they
+    share the root); the two branches then add to x one after the other."""
     graph_safe = True      # launches depend on device memory only
 
     def __init__(self, mixer_norm: Norm, mixer: Mixer, ffn_norm: Norm | None, ffn: FeedForward | None):
@@ -61,15 +62,39 @@ class ParallelBlock(Block):
     def children(self):
         return [p for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn) if p is not None]
 
+    def _shared_root(self):
+        """The two norms as (NormRef, NormRef) if they are RMS norms with one eps over the same width,
+        so that one pass over a row serves both; else None."""
+        if self.ffn is None:
+            return None
+        a, c = norm_ref_of(self.mixer_norm), norm_ref_of(self.ffn_norm)
+        if a is None or c is None or a.eps != c.eps or a.weight.shape != c.weight.shape:
+            return None
+        return a, c
+
     def first_norm(self):
+        """The norm that the block before may have prepared: the mixer's, unless one kernel takes
+        both norms of this block."""
+        if self.ffn is not None and all(getattr(n, "weight", None) is not None for n in (self.mixer_norm, self.ffn_norm)) and self._shared_root():
+            return None
         return self.mixer_norm
 
     def emit(self, b, x: int, after=None, after_when: int = 0) -> None:
-        from ..engine.program import Rows
-        src = self.mixer_norm.emit(b, x)
+        from ..engine.program import _DT, Rows
+        from .calls import RmsPairArgs, emit_library_call
         if self.ffn is None:
-            self.mixer.emit(b, src, x, after, after_when)
+            self.mixer.emit(b, self.mixer_norm.emit(b, x), x, after, after_when)
             return
+        pair = self._shared_root()
+        if pair is not None:
+            first = b.buffer("norm.out", self.mixer_norm.size, b.dtype)
+            second = b.buffer("norm.out.second", self.ffn_norm.size, b.dtype)
+            emit_library_call(b, "rms_pair", RmsPairArgs(b._ptr(pair[0].weight), b._ptr(pair[1].weight), self.mixer_norm.size, _DT[b.dtype],
+                                                        pair[0].eps), first, inp=x, extra=[second])
+            self.mixer.emit(b, Rows(first), x, None, 0)
+            self.ffn.emit(b, Rows(second), x, after, after_when)
+            return
+        src = self.mixer_norm.emit(b, x)
         second = self.ffn_norm.emit(b, x)
         if second.norm is not None:         # rows of their own: the first norm's place is in use until the mixer has read it
             second = Rows(b.buffer("norm.out.second", self.ffn_norm.size, b.dtype), second.norm, second.x)

@@ -119,6 +119,10 @@ class AddRowsArgs(Structure):
     _fields_ = [("vec", c_void_p), ("width", c_int32)]
 
 
+class RmsPairArgs(Structure):
+    _fields_ = [("w_a", c_void_p), ("w_b", c_void_p), ("width", c_int32), ("out_dtype", c_int32), ("eps", c_float)]
+
+
 class MapDifferenceArgs(Structure):
     _fields_ = [("heads", c_int32), ("vdim", c_int32), ("out_dtype", c_int32), ("lam", c_float), ("eps", c_float), ("mult", c_float)]
 
