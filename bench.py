@@ -281,9 +281,9 @@ def _kekelix_pair(width: int, heads: int, stretch: int, experts: int, top: int, 
     windows are `stretch` keys."""
     mlp = dict(kind="moe", router=dict(experts=experts, top=top), expert=dict(ff=width, limit=7.0))
     G = max(heads // 4, 1)
-    kinds = [dict(type="attention", mixer=dict(heads=heads, kv_heads=G, dim=64, vdim=128, scale=64 ** -0.5, diff=0.3), mlp=mlp),
+    kinds = [dict(type="attention", mixer=dict(heads=heads, kv_heads=G, dim=64, vdim=128, scale=64 ** -0.5, diff=0.25), mlp=mlp),
              dict(type="attention_3", mixer=dict(heads=heads, kv_heads=G, dim=128, vdim=128, scale=128 ** -0.5,
-                                                 rot=dict(base=250000.0, dims=64), mask=dict(size=stretch)), mlp=mlp),
+                                                 rot=dict(base=500000.0, dims=64), mask=dict(size=stretch)), mlp=mlp),
              dict(type="attention_2", mixer=dict(heads=heads, kv_heads=G, dim=128, vdim=128, scale=128 ** -0.5,
                                                  rot=dict(base=10000.0, dims=64, scaling=dict(factor=8.0, original=4096, fast=32.0, slow=1.0))),
                   mlp=mlp)]

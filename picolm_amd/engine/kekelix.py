@@ -55,6 +55,8 @@ def build_kekelix(cfg: KekelixConfig) -> DecoderModel:
     n_layers = len(blocks)
     if cfg.loop is not None:
         blocks += [LoopSum("loop.step", D, cfg.loop.times, t) for t in range(cfg.loop.times)]
+    else:
+        unused.append(TensorSpec("loop.step", (-1, D), optional=True, init=None))       # a checkpoint may carry the passes' vectors all the same
     order = []
     for i, t, first in cfg.layer_runs():
         if first:

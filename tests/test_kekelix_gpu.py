@@ -73,6 +73,7 @@ ALONE = {
     "two maps a head, a KV head a head": one_layer(kt.difference(3, 3, 10, 6, 0.4, 0.8)),
     "two maps a head, one head": one_layer(kt.difference(1, 1, 5, 7, 0.5, 0.05)),
     "two maps, cached keys of 64 and values of 96": one_layer(kt.difference(8, 2, 32, 96, 0.2, 0.3), width=64),       # the matrix-core kernel in bfloat16
+    "two maps, cached keys of 96 and values of 128": one_layer(kt.difference(6, 3, 48, 128, 0.15, 0.45), width=64),
     "two maps, cached keys of 128 and values of 64": one_layer(kt.difference(4, 4, 64, 64, 0.15, 0.5), width=64),
     "two maps, cached keys of 320": one_layer(kt.difference(2, 1, 160, 24, 0.1, 0.3), width=64),                      # beyond what a thread's registers hold of a key
     "biases, a part turned, one more in the denominator": one_layer(kt.sinked(6, 2, 20, 12, 0.25, 8, 500.0)),
@@ -385,7 +386,7 @@ def test_one_far_key_among_hundreds(kind, dim, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("size,dim", [(70, 40), (64, 40), (129, 40), (2, 40), (33, 64), (100, 64), (200, 64)])
+@pytest.mark.parametrize("size,dim", [(70, 40), (64, 40), (129, 40), (2, 40), (33, 64), (100, 64), (190, 64)])
 def test_a_key_just_inside_and_just_outside_a_stretch(size, dim, dtype):
     """The partner of the last token stands at the first place of the last token's stretch and at
     the place before it: seen, the logits rest on it; not seen, they are what they are without it.
