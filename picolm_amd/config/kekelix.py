@@ -76,8 +76,11 @@ class KekelixMixer:
             mask = _integer(_object(d, where, "mask"), where + "mask.", "size")
         dim = _integer(d, where, "dim")
         # where the values are the keys they have the keys' size, whatever `vdim` says
-        c = KekelixMixer(kind, _integer(d, where, "heads"), _integer(d, where, "kv_heads"), dim,
-                         dim if kind == "attention_3" else _integer(d, where, "vdim"), _number(d, where, "scale"), diff, rot, mask or 0)
+        heads = _integer(d, where, "heads")
+        # (a configuration that leaves them out: a KV head a head, and the usual 1 / sqrt(dim))
+        c = KekelixMixer(kind, heads, _integer(d, where, "kv_heads", heads), dim,
+                         dim if kind == "attention_3" else _integer(d, where, "vdim"), _number(d, where, "scale", dim ** -0.5), diff, rot,
+                         mask or 0)
         if c.heads % c.kv_heads:
             raise ConfigError(f"{where}kv_heads: {c.kv_heads} does not divide heads = {c.heads}")
         key = 2 * c.dim if kind == "attention" else c.dim          # both maps' keys of a token are cached side by side

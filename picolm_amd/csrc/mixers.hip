@@ -171,8 +171,7 @@ extern "C" int picolm_call_sink_attention(void* user, const picolm_step_view* v)
     dim3 grid(v->n_tokens, v->kv_writes ? (H + G) * maps + G : H * maps);
     const bool mfma = dt == PICOLM_BF16 && picolm_attn_plain_mfma_takes(d, dv);      // then the pages are in the matrix-core kernel's order
     QkPrepare p = {in, a->in_stride, a->q_off, a->k_off, a->v_off, a->q_norm, a->k_norm, a->eps, a->unit_qk, a->in_bias, a->cos_table,
-                   a->sin_table, a->table_positions, a->rot_dims, a->rot_half, v->tok_pos, v->write_pages, H, G, d, dv, maps,
-                   dt == PICOLM_BF16 && mfma};
+                   a->sin_table, a->table_positions, a->rot_dims, a->rot_half, v->tok_pos, v->write_pages, H, G, d, dv, maps, mfma};
     if (dt == PICOLM_F32)
         qk_norm_store_kernel<float><<<grid, WAVE, 0, v->stream>>>(p, (float*)v->extra[0], (float*)v->k_pages, (float*)v->v_pages);
     else

@@ -75,9 +75,7 @@ class ParallelBlock(Block):
     def first_norm(self):
         """The norm that the block before may have prepared: the mixer's, unless one kernel takes
         both norms of this block."""
-        if self.ffn is not None and all(getattr(n, "weight", None) is not None for n in (self.mixer_norm, self.ffn_norm)) and self._shared_root():
-            return None
-        return self.mixer_norm
+        return None if self._shared_root() else self.mixer_norm
 
     def emit(self, b, x: int, after=None, after_when: int = 0) -> None:
         from ..engine.program import _DT, Rows
